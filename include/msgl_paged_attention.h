@@ -1,0 +1,162 @@
+/*
+ * msgl_paged_attention.h -- C ABI of the MI355X (gfx950) paged-attention hot path.
+ *
+ * Three operators, the ones the reference's `mini_sglang_mlx_kernel._ext` module
+ * binds for this path (mini-sglang-mlx-kernel/csrc/bindings.cpp:27-55):
+ *
+ *   store_kv_cache            in-place scatter of new K/V rows into the slot-indexed pools
+ *   paged_decode_attention    GQA split-K decode over slots gathered through kv_indices
+ *   paged_prefill_attention   extend attention (causal / full / window / bidirectional+window)
+ *
+ * Conventions shared by every entry point
+ *   - every pointer is a DEVICE pointer in the address space of the current HIP
+ *     device; `stream` is a hipStream_t passed as void* (NULL = the null stream);
+ *   - the library never allocates, frees, retains or synchronises: launches are
+ *     stream-ordered and the call returns as soon as they are enqueued;
+ *   - pools are (num_slots, num_kv_heads, head_dim) with the two inner dimensions
+ *     contiguous; `*_stride0` is the distance between consecutive slots in ELEMENTS;
+ *   - q / out are contiguous (rows, num_q_heads, head_dim);
+ *   - index arrays are int32; kv_indices holds one pool slot per token (the
+ *     reference's token-granular contract);
+ *   - return value: MSGL_OK (0) or a negative MSGL_ERR_* code; no exception and
+ *     no abort crosses this boundary.  msgl_strerror() gives the text.
+ */
+#ifndef MSGL_PAGED_ATTENTION_H
+#define MSGL_PAGED_ATTENTION_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#if defined(__GNUC__)
+#define MSGL_API __attribute__((visibility("default")))
+#else
+#define MSGL_API
+#endif
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* element types of q / k / v / pools / out */
+#define MSGL_DTYPE_BF16 0
+#define MSGL_DTYPE_F16 1
+
+#define MSGL_OK 0
+#define MSGL_ERR_NULL_POINTER (-1)      /* a required pointer is NULL */
+#define MSGL_ERR_HEAD_DIM (-2)          /* head_dim is not 128 or 256 */
+#define MSGL_ERR_HEAD_RATIO (-3)        /* num_q_heads is not a multiple of num_kv_heads */
+#define MSGL_ERR_GROUP_TOO_LARGE (-4)   /* decode: num_q_heads / num_kv_heads > 16 */
+#define MSGL_ERR_DTYPE (-5)             /* unsupported element type for this operator */
+#define MSGL_ERR_BATCH (-6)             /* prefill: batch <= 0 */
+#define MSGL_ERR_WINDOW (-7)            /* prefill: sliding_window_size < 0 */
+#define MSGL_ERR_WORKSPACE (-8)         /* workspace missing or smaller than *_workspace_bytes() */
+#define MSGL_ERR_SHAPE (-9)             /* negative size, stride smaller than a row, ... */
+#define MSGL_ERR_ALIGNMENT (-10)        /* pointer or stride not aligned for the vector width used */
+#define MSGL_ERR_LAUNCH (-11)           /* the HIP runtime refused a launch (hipGetLastError) */
+#define MSGL_ERR_HEAD_DIM_MULT4 (-12)   /* store: head_dim is not a multiple of 4 */
+
+/* Library version: major*10000 + minor*100 + patch. */
+MSGL_API int msgl_version(void);
+
+/* Static, never-NULL description of a return code. */
+MSGL_API const char* msgl_strerror(int code);
+
+/*
+ * store_kv_cache -- replaces mini_sglang_mlx::store_kv_cache
+ * (mini-sglang-mlx-kernel/csrc/store_kv_cache.cpp:14-107, kernel store_kv_cache.metal:7-31):
+ *     k_cache[indices[r], :, :] = k[r, :, :];  v_cache[indices[r], :, :] = v[r, :, :]
+ * Bit copy of `elem_bytes`-wide elements (2 for bf16/f16).  The caller guarantees
+ * indices are unique and inside [0, num_slots); duplicate indices race, as in the
+ * reference.  Unlike the reference, which applies k's strides to v and k_cache's to
+ * v_cache (store_kv_cache.cpp:65-66), all four leading strides are taken explicitly.
+ * `length == 0` is a no-op.
+ */
+MSGL_API int msgl_store_kv_cache(void* k_cache, void* v_cache, const int32_t* indices,
+                        const void* k, const void* v,
+                        int64_t length, int64_t num_kv_heads, int64_t head_dim,
+                        int64_t num_slots,
+                        int64_t k_cache_stride0, int64_t v_cache_stride0,
+                        int64_t k_stride0, int64_t v_stride0,
+                        int32_t elem_bytes, void* stream);
+
+/*
+ * Workspace (bytes) that msgl_paged_decode_attention needs for these sizes.
+ * `total_kv` is the length of kv_indices.  Replaces the per-call att_out/att_lse
+ * allocation of PagedDecodeAttention::eval_gpu (paged_decode_attention.cpp:118-129).
+ */
+MSGL_API size_t msgl_paged_decode_workspace_bytes(int64_t batch, int64_t total_kv,
+                                         int64_t num_q_heads, int64_t num_kv_heads,
+                                         int64_t head_dim);
+
+/*
+ * paged_decode_attention -- replaces mini_sglang_mlx::paged_decode_attention
+ * (paged_decode_attention.cpp:15-73; kernels paged_decode_attention.metal:313-586).
+ *   q   (batch, num_q_heads, head_dim)      out (batch, num_q_heads, head_dim)
+ *   kv_indptr (batch+1)   kv_indices (total_kv)   num_kv_splits (batch)
+ * Request b attends to all kv_indptr[b+1]-kv_indptr[b] tokens listed for it.
+ * The KV range of a request is cut into fixed-size chunks chosen for MI355X
+ * occupancy; partial results are merged by log-sum-exp.  The result does not
+ * depend on the split, so `num_kv_splits` / `max_kv_splits` (the reference's
+ * split hints, backend.py:304-307) are accepted and validated but do not steer
+ * the cut.  A request with no tokens gets zeros (the reference leaves its rows
+ * unwritten, paged_decode_attention.metal:354).
+ */
+MSGL_API int msgl_paged_decode_attention(const void* q, const void* k_cache, const void* v_cache,
+                                const int32_t* kv_indptr, const int32_t* kv_indices,
+                                const int32_t* num_kv_splits, void* out,
+                                void* workspace, size_t workspace_bytes,
+                                int64_t batch, int64_t total_kv,
+                                int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim,
+                                int64_t num_slots,
+                                int64_t k_cache_stride0, int64_t v_cache_stride0,
+                                float sm_scale, int32_t max_kv_splits,
+                                int32_t dtype, void* stream);
+
+/* Workspace (bytes) that msgl_paged_prefill_attention needs for these sizes. */
+MSGL_API size_t msgl_paged_prefill_workspace_bytes(int64_t batch, int64_t total_q, int64_t total_kv,
+                                          int64_t num_q_heads, int64_t num_kv_heads,
+                                          int64_t head_dim, int64_t max_len_extend);
+
+/*
+ * paged_prefill_attention -- replaces mini_sglang_mlx::paged_prefill_attention
+ * (paged_prefill_attention.cpp:18-87; kernel paged_prefill_attention.metal:382-640).
+ *   q   (total_q, num_q_heads, head_dim)    out (total_q, num_q_heads, head_dim)
+ *   qo_indptr (batch+1)  kv_indptr (batch+1)  kv_indices (total_kv)  prefix_lens (batch)
+ * Query i of request b sits at position prefix_lens[b] + i; key j (index in the
+ * request's kv stream) is visible iff
+ *     (is_cross_attention || j <= qpos) && (window == 0 || j >= qpos - window + 1)
+ * (paged_prefill_attention.metal:339-347).  A query with no visible key gets zeros
+ * (:627-630).  Requests whose query length exceeds `max_len_extend` are computed only
+ * for their first max_len_extend queries, as in the reference's grid
+ * (paged_prefill_attention.cpp:152-159).  Short query blocks (speculative verify,
+ * draft proposal) are routed to the bandwidth-bound split-K kernel, long ones to
+ * the MFMA tile kernel; same arguments, same result.
+ */
+MSGL_API int msgl_paged_prefill_attention(const void* q, const void* k_cache, const void* v_cache,
+                                 const int32_t* qo_indptr, const int32_t* kv_indptr,
+                                 const int32_t* kv_indices, const int32_t* prefix_lens,
+                                 void* out, void* workspace, size_t workspace_bytes,
+                                 int64_t batch, int64_t total_q, int64_t total_kv,
+                                 int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim,
+                                 int64_t num_slots,
+                                 int64_t k_cache_stride0, int64_t v_cache_stride0,
+                                 float sm_scale, int32_t max_len_extend,
+                                 int32_t is_cross_attention, int32_t sliding_window_size,
+                                 int32_t dtype, void* stream);
+
+/*
+ * Tuning knobs, for benchmarking only (0 = built-in heuristic).  Process-wide,
+ * read at launch time; not part of the reference surface.
+ *   MSGL_TUNE_DECODE_CHUNK   tokens per split-K work item in decode (multiple of 32)
+ *   MSGL_TUNE_SMALLQ_CHUNK   same for the short-query route of prefill
+ *   MSGL_TUNE_SMALLQ_MAXCOLS largest q_len*group routed to the split-K kernel
+ */
+#define MSGL_TUNE_DECODE_CHUNK 0
+#define MSGL_TUNE_SMALLQ_CHUNK 1
+#define MSGL_TUNE_SMALLQ_MAXCOLS 2
+MSGL_API int msgl_set_tuning(int32_t knob, int64_t value);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MSGL_PAGED_ATTENTION_H */

@@ -1,0 +1,247 @@
+// extern "C" entry points of libmsgl_paged_attention.so: argument checks and routing.
+// The checks mirror the reference's host functions (paged_decode_attention.cpp:25-62,
+// paged_prefill_attention.cpp:31-76, store_kv_cache.cpp:22-63) as far as raw pointers
+// and sizes can express them; rank and dtype-equality checks live in the Python shim.
+#include <atomic>
+
+#include "msgl_internal.h"
+
+namespace {
+
+std::atomic<int64_t> g_tune[3] = {{0}, {0}, {0}};
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+int check_common(const void* q, const void* k_cache, const void* v_cache, const void* out,
+                 int64_t n_q, int64_t n_kv, int64_t d, int64_t k_stride0, int64_t v_stride0,
+                 int32_t dtype, const char*) {
+  if (d != 128 && d != 256) return MSGL_ERR_HEAD_DIM;
+  if (n_q <= 0 || n_kv <= 0) return MSGL_ERR_SHAPE;
+  if (n_q % n_kv != 0) return MSGL_ERR_HEAD_RATIO;
+  if (dtype != MSGL_DTYPE_BF16) return MSGL_ERR_DTYPE;
+  if (k_stride0 < n_kv * d || v_stride0 < n_kv * d) return MSGL_ERR_SHAPE;
+  if (!q || !k_cache || !v_cache || !out) return MSGL_ERR_NULL_POINTER;
+  // 16-byte row segments are the unit of every load and store
+  if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || !aligned16(out) ||
+      k_stride0 % 8 != 0 || v_stride0 % 8 != 0)
+    return MSGL_ERR_ALIGNMENT;
+  return MSGL_OK;
+}
+
+int32_t decode_chunk(int64_t total_kv, int64_t n_kv, int64_t group) {
+  const int64_t t = g_tune[MSGL_TUNE_DECODE_CHUNK].load();
+  if (t >= 32) return (int32_t)(t / 32 * 32);
+  return msgl::splitkv_default_chunk(total_kv, n_kv, group);
+}
+int32_t smallq_chunk(int64_t total_kv, int64_t n_kv, int64_t cols) {
+  const int64_t t = g_tune[MSGL_TUNE_SMALLQ_CHUNK].load();
+  if (t >= 32) return (int32_t)(t / 32 * 32);
+  return msgl::splitkv_default_chunk(total_kv, n_kv, cols);
+}
+int64_t smallq_max_cols() {
+  const int64_t t = g_tune[MSGL_TUNE_SMALLQ_MAXCOLS].load();
+  if (t < 0) return 0;  // negative: never take the split-K route
+  if (t > 0) return t < msgl::kSplitKvMaxCols ? t : msgl::kSplitKvMaxCols;
+  return msgl::kSplitKvMaxCols;
+}
+
+}  // namespace
+
+extern "C" {
+
+int msgl_version(void) { return 100; }
+
+const char* msgl_strerror(int code) {
+  switch (code) {
+    case MSGL_OK: return "ok";
+    case MSGL_ERR_NULL_POINTER: return "a required pointer is NULL";
+    case MSGL_ERR_HEAD_DIM: return "head_dim must be 128 or 256";
+    case MSGL_ERR_HEAD_RATIO: return "num_q_heads must be a multiple of num_kv_heads";
+    case MSGL_ERR_GROUP_TOO_LARGE: return "only q_heads/kv_heads <= 16 is supported";
+    case MSGL_ERR_DTYPE: return "unsupported dtype";
+    case MSGL_ERR_BATCH: return "batch must be > 0";
+    case MSGL_ERR_WINDOW: return "sliding_window_size must be >= 0";
+    case MSGL_ERR_WORKSPACE: return "workspace missing or too small";
+    case MSGL_ERR_SHAPE: return "invalid size or stride";
+    case MSGL_ERR_ALIGNMENT: return "pointer or stride not aligned to the vector width";
+    case MSGL_ERR_LAUNCH: return "HIP kernel launch failed";
+    case MSGL_ERR_HEAD_DIM_MULT4: return "head_dim must be a multiple of 4";
+    default: return "unknown error code";
+  }
+}
+
+int msgl_set_tuning(int32_t knob, int64_t value) {
+  if (knob < 0 || knob > 2) return MSGL_ERR_SHAPE;
+  g_tune[knob].store(value);
+  return MSGL_OK;
+}
+
+int msgl_store_kv_cache(void* k_cache, void* v_cache, const int32_t* indices, const void* k,
+                        const void* v, int64_t length, int64_t num_kv_heads, int64_t head_dim,
+                        int64_t num_slots, int64_t k_cache_stride0, int64_t v_cache_stride0,
+                        int64_t k_stride0, int64_t v_stride0, int32_t elem_bytes, void* stream) {
+  if (length < 0 || num_kv_heads <= 0 || head_dim <= 0 || num_slots < 0) return MSGL_ERR_SHAPE;
+  if (elem_bytes != 2 && elem_bytes != 4) return MSGL_ERR_DTYPE;
+  if (head_dim % 4 != 0) return MSGL_ERR_HEAD_DIM_MULT4;  // store_kv_cache.cpp:49-52
+  const int64_t row = num_kv_heads * head_dim;
+  if (k_cache_stride0 < row || v_cache_stride0 < row || k_stride0 < row || v_stride0 < row)
+    return MSGL_ERR_SHAPE;
+  if (length == 0) return MSGL_OK;
+  if (!k_cache || !v_cache || !indices || !k || !v) return MSGL_ERR_NULL_POINTER;
+  return msgl::launch_store_kv_cache(k_cache, v_cache, indices, k, v, length, row * elem_bytes,
+                                     k_cache_stride0 * elem_bytes, v_cache_stride0 * elem_bytes,
+                                     k_stride0 * elem_bytes, v_stride0 * elem_bytes,
+                                     static_cast<hipStream_t>(stream));
+}
+
+size_t msgl_paged_decode_workspace_bytes(int64_t batch, int64_t total_kv, int64_t num_q_heads,
+                                         int64_t num_kv_heads, int64_t head_dim) {
+  if (batch <= 0 || total_kv < 0 || num_q_heads <= 0 || num_kv_heads <= 0 ||
+      num_q_heads % num_kv_heads != 0)
+    return 0;
+  const int64_t group = num_q_heads / num_kv_heads;
+  return msgl::splitkv_workspace_bytes(batch, total_kv, num_q_heads, num_kv_heads, head_dim, 1,
+                                       decode_chunk(total_kv, num_kv_heads, group));
+}
+
+int msgl_paged_decode_attention(const void* q, const void* k_cache, const void* v_cache,
+                                const int32_t* kv_indptr, const int32_t* kv_indices,
+                                const int32_t* num_kv_splits, void* out, void* workspace,
+                                size_t workspace_bytes, int64_t batch, int64_t total_kv,
+                                int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim,
+                                int64_t num_slots, int64_t k_cache_stride0,
+                                int64_t v_cache_stride0, float sm_scale, int32_t max_kv_splits,
+                                int32_t dtype, void* stream) {
+  if (batch < 0 || total_kv < 0 || num_slots < 0) return MSGL_ERR_SHAPE;
+  if (batch == 0) return MSGL_OK;
+  int rc = check_common(q, k_cache, v_cache, out, num_q_heads, num_kv_heads, head_dim,
+                        k_cache_stride0, v_cache_stride0, dtype, "paged_decode_attention");
+  if (rc != MSGL_OK) return rc;
+  const int64_t group = num_q_heads / num_kv_heads;
+  if (group > 16) return MSGL_ERR_GROUP_TOO_LARGE;  // paged_decode_attention.cpp:54-57
+  if (!kv_indptr || !num_kv_splits || (total_kv > 0 && !kv_indices)) return MSGL_ERR_NULL_POINTER;
+  (void)max_kv_splits;  // split hints do not steer the cut (result is split-invariant)
+  const int32_t chunk = decode_chunk(total_kv, num_kv_heads, group);
+  const size_t need = msgl::splitkv_workspace_bytes(batch, total_kv, num_q_heads, num_kv_heads,
+                                                    head_dim, 1, chunk);
+  if (!workspace || workspace_bytes < need || !aligned16(workspace)) return MSGL_ERR_WORKSPACE;
+  msgl::SplitKvArgs a{};
+  a.q = q;
+  a.k_cache = k_cache;
+  a.v_cache = v_cache;
+  a.kv_indptr = kv_indptr;
+  a.kv_indices = kv_indices;
+  a.qo_indptr = nullptr;
+  a.prefix_lens = nullptr;
+  a.out = out;
+  a.workspace = workspace;
+  a.batch = batch;
+  a.total_kv = total_kv;
+  a.n_q = num_q_heads;
+  a.n_kv = num_kv_heads;
+  a.head_dim = head_dim;
+  a.k_stride0 = k_cache_stride0;
+  a.v_stride0 = v_cache_stride0;
+  a.sm_scale = sm_scale;
+  a.max_len_extend = 1;
+  a.is_cross = 0;
+  a.window = 0;
+  a.chunk = chunk;
+  return msgl::launch_splitkv(a, static_cast<hipStream_t>(stream));
+}
+
+static bool use_splitkv_route(int64_t group, int64_t max_len_extend) {
+  return max_len_extend >= 1 && group * max_len_extend <= smallq_max_cols();
+}
+
+size_t msgl_paged_prefill_workspace_bytes(int64_t batch, int64_t total_q, int64_t total_kv,
+                                          int64_t num_q_heads, int64_t num_kv_heads,
+                                          int64_t head_dim, int64_t max_len_extend) {
+  (void)total_q;
+  if (batch <= 0 || total_kv < 0 || num_q_heads <= 0 || num_kv_heads <= 0 ||
+      num_q_heads % num_kv_heads != 0)
+    return 0;
+  const int64_t group = num_q_heads / num_kv_heads;
+  if (!use_splitkv_route(group, max_len_extend)) return 0;
+  return msgl::splitkv_workspace_bytes(
+      batch, total_kv, num_q_heads, num_kv_heads, head_dim, max_len_extend,
+      smallq_chunk(total_kv, num_kv_heads, group * max_len_extend));
+}
+
+int msgl_paged_prefill_attention(const void* q, const void* k_cache, const void* v_cache,
+                                 const int32_t* qo_indptr, const int32_t* kv_indptr,
+                                 const int32_t* kv_indices, const int32_t* prefix_lens, void* out,
+                                 void* workspace, size_t workspace_bytes, int64_t batch,
+                                 int64_t total_q, int64_t total_kv, int64_t num_q_heads,
+                                 int64_t num_kv_heads, int64_t head_dim, int64_t num_slots,
+                                 int64_t k_cache_stride0, int64_t v_cache_stride0, float sm_scale,
+                                 int32_t max_len_extend, int32_t is_cross_attention,
+                                 int32_t sliding_window_size, int32_t dtype, void* stream) {
+  if (head_dim != 128 && head_dim != 256) return MSGL_ERR_HEAD_DIM;
+  if (num_q_heads <= 0 || num_kv_heads <= 0) return MSGL_ERR_SHAPE;
+  if (num_q_heads % num_kv_heads != 0) return MSGL_ERR_HEAD_RATIO;
+  if (sliding_window_size < 0) return MSGL_ERR_WINDOW;  // paged_prefill_attention.cpp:67-70
+  if (batch <= 0) return MSGL_ERR_BATCH;                // :74-77
+  if (total_q < 0 || total_kv < 0 || num_slots < 0) return MSGL_ERR_SHAPE;
+  if (total_q == 0 || max_len_extend <= 0) return MSGL_OK;
+  int rc = check_common(q, k_cache, v_cache, out, num_q_heads, num_kv_heads, head_dim,
+                        k_cache_stride0, v_cache_stride0, dtype, "paged_prefill_attention");
+  if (rc != MSGL_OK) return rc;
+  if (!qo_indptr || !kv_indptr || !prefix_lens || (total_kv > 0 && !kv_indices))
+    return MSGL_ERR_NULL_POINTER;
+  const int64_t group = num_q_heads / num_kv_heads;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (use_splitkv_route(group, max_len_extend)) {
+    const int32_t chunk = smallq_chunk(total_kv, num_kv_heads, group * max_len_extend);
+    const size_t need = msgl::splitkv_workspace_bytes(batch, total_kv, num_q_heads, num_kv_heads,
+                                                      head_dim, max_len_extend, chunk);
+    if (!workspace || workspace_bytes < need || !aligned16(workspace)) return MSGL_ERR_WORKSPACE;
+    msgl::SplitKvArgs a{};
+    a.q = q;
+    a.k_cache = k_cache;
+    a.v_cache = v_cache;
+    a.kv_indptr = kv_indptr;
+    a.kv_indices = kv_indices;
+    a.qo_indptr = qo_indptr;
+    a.prefix_lens = prefix_lens;
+    a.out = out;
+    a.workspace = workspace;
+    a.batch = batch;
+    a.total_kv = total_kv;
+    a.n_q = num_q_heads;
+    a.n_kv = num_kv_heads;
+    a.head_dim = head_dim;
+    a.k_stride0 = k_cache_stride0;
+    a.v_stride0 = v_cache_stride0;
+    a.sm_scale = sm_scale;
+    a.max_len_extend = max_len_extend;
+    a.is_cross = is_cross_attention ? 1 : 0;
+    a.window = sliding_window_size;
+    a.chunk = chunk;
+    return msgl::launch_splitkv(a, s);
+  }
+  msgl::PrefillArgs a{};
+  a.q = q;
+  a.k_cache = k_cache;
+  a.v_cache = v_cache;
+  a.qo_indptr = qo_indptr;
+  a.kv_indptr = kv_indptr;
+  a.kv_indices = kv_indices;
+  a.prefix_lens = prefix_lens;
+  a.out = out;
+  a.batch = batch;
+  a.total_q = total_q;
+  a.total_kv = total_kv;
+  a.n_q = num_q_heads;
+  a.n_kv = num_kv_heads;
+  a.head_dim = head_dim;
+  a.k_stride0 = k_cache_stride0;
+  a.v_stride0 = v_cache_stride0;
+  a.sm_scale = sm_scale;
+  a.max_len_extend = max_len_extend;
+  a.is_cross = is_cross_attention ? 1 : 0;
+  a.window = sliding_window_size;
+  return msgl::launch_prefill_tile(a, s);
+}
+
+}  // extern "C"

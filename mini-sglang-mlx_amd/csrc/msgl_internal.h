@@ -1,0 +1,64 @@
+// Host-side declarations shared by the translation units of libmsgl_paged_attention.so.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "../../include/msgl_paged_attention.h"
+
+namespace msgl {
+
+// ---- store_kv_cache.hip ------------------------------------------------------------
+int launch_store_kv_cache(void* k_cache, void* v_cache, const int32_t* indices, const void* k,
+                          const void* v, int64_t length, int64_t row_bytes,
+                          int64_t k_cache_stride_bytes, int64_t v_cache_stride_bytes,
+                          int64_t k_stride_bytes, int64_t v_stride_bytes, hipStream_t stream);
+
+// ---- paged_splitkv.hip -------------------------------------------------------------
+// One description serves decode (qo_indptr == nullptr: one query per request, every key
+// visible) and the short-query route of prefill (speculative verify / draft proposal).
+struct SplitKvArgs {
+  const void* q;
+  const void* k_cache;
+  const void* v_cache;
+  const int32_t* kv_indptr;
+  const int32_t* kv_indices;
+  const int32_t* qo_indptr;    // nullptr for decode
+  const int32_t* prefix_lens;  // nullptr for decode
+  void* out;
+  void* workspace;
+  int64_t batch, total_kv, n_q, n_kv, head_dim;
+  int64_t k_stride0, v_stride0;  // elements
+  float sm_scale;
+  int32_t max_len_extend;  // 1 for decode
+  int32_t is_cross, window;
+  int32_t chunk;  // tokens per work item, multiple of 32
+};
+// largest q_len * group the split-K kernel is instantiated for
+constexpr int kSplitKvMaxCols = 64;
+int splitkv_default_chunk(int64_t total_kv, int64_t n_kv, int64_t cols);
+size_t splitkv_workspace_bytes(int64_t batch, int64_t total_kv, int64_t n_q, int64_t n_kv,
+                               int64_t head_dim, int64_t max_len_extend, int32_t chunk);
+int launch_splitkv(const SplitKvArgs& a, hipStream_t stream);
+
+// ---- paged_prefill.hip -------------------------------------------------------------
+struct PrefillArgs {
+  const void* q;
+  const void* k_cache;
+  const void* v_cache;
+  const int32_t* qo_indptr;
+  const int32_t* kv_indptr;
+  const int32_t* kv_indices;
+  const int32_t* prefix_lens;
+  void* out;
+  int64_t batch, total_q, total_kv, n_q, n_kv, head_dim;
+  int64_t k_stride0, v_stride0;  // elements
+  float sm_scale;
+  int32_t max_len_extend;
+  int32_t is_cross, window;
+};
+int launch_prefill_tile(const PrefillArgs& a, hipStream_t stream);
+
+inline int check_launch() { return hipGetLastError() == hipSuccess ? MSGL_OK : MSGL_ERR_LAUNCH; }
+
+}  // namespace msgl

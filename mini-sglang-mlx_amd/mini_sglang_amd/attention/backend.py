@@ -1,0 +1,169 @@
+"""Attention backend of the path on torch-ROCm
+(reference: mini_sglang_mlx/attention/backend.py:15-307).
+
+``AttnBackend.forward`` stores the new K/V rows first and then attends through the slot
+lists, so the new tokens are read back from the pool exactly like cached ones
+(backend.py:139-141).  Metadata are int32 CSR arrays; ``kv_indices`` holds one pool slot
+per token.  The builders keep the reference's formulas and keyword overrides (virtual
+extend windows for speculative verify, backend.py:205-293).
+"""
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass
+from typing import List, Optional, Sequence
+
+import torch
+
+from mini_sglang_amd_kernel import paged_decode_attention, paged_prefill_attention
+
+MAX_KV_SPLITS = 32
+
+
+@dataclass
+class BaseAttnMetadata:
+    positions: torch.Tensor
+
+    def get_last_indices(self, bs: int) -> torch.Tensor:
+        raise NotImplementedError
+
+
+@dataclass
+class PrefillMetadata(BaseAttnMetadata):
+    """Several new query tokens per sequence on top of a cached prefix (backend.py:26-41)."""
+
+    qo_indptr: torch.Tensor  # (batch + 1,) int32
+    kv_indptr: torch.Tensor  # (batch + 1,) int32
+    kv_indices: torch.Tensor  # (total_kv,) int32 pool slots
+    prefix_lens: torch.Tensor  # (batch,) int32
+    max_len_extend: int
+
+    def get_last_indices(self, bs: int) -> torch.Tensor:
+        return self.qo_indptr[1 : 1 + bs] - 1
+
+
+@dataclass
+class DecodeMetadata(BaseAttnMetadata):
+    """One new query token per sequence (backend.py:44-58)."""
+
+    kv_indptr: torch.Tensor  # (batch + 1,) int32
+    kv_indices: torch.Tensor  # (total_kv,) int32 pool slots
+    num_kv_splits: torch.Tensor  # (batch,) int32
+    max_kv_splits: int
+
+    def get_last_indices(self, bs: int) -> torch.Tensor:
+        return torch.arange(bs, dtype=torch.int32, device=self.kv_indptr.device)
+
+
+AttnMetadata = PrefillMetadata | DecodeMetadata
+
+
+class AttnBackend:
+    """Paged attention backend for MI355X using the msgl HIP kernels.
+
+    ``config`` needs ``head_dim``; ``kvcache`` is a ``BaseKVCache``; ``page_table`` is the
+    ``(max_running_req + 1, max_seq_len)`` int32 slot table the scheduler fills.
+    """
+
+    def __init__(self, config, kvcache, page_table: torch.Tensor) -> None:
+        self.config = config
+        self.kvcache = kvcache
+        self.page_table = page_table
+        self.sm_scale = 1.0 / math.sqrt(config.head_dim)
+
+    def forward(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, layer_id: int, batch, *,
+                is_cross_attention: bool = False, sliding_window_size: int = 0) -> torch.Tensor:
+        """Write the new K/V rows at ``batch.out_loc`` and run paged attention.
+
+        The two flags select one of four masks on the prefill path (backend.py:112-127):
+        causal, full, causal + window, bidirectional + window.  Decode rejects both.
+        """
+        assert sliding_window_size >= 0, (
+            f"sliding_window_size must be >= 0, got {sliding_window_size}"
+        )
+        metadata = batch.attn_metadata
+        self.kvcache.store_kv(k, v, batch.out_loc, layer_id)
+        k_cache = self.kvcache.k_cache(layer_id)
+        v_cache = self.kvcache.v_cache(layer_id)
+
+        if isinstance(metadata, PrefillMetadata):
+            return paged_prefill_attention(
+                q, k_cache, v_cache, metadata.qo_indptr, metadata.kv_indptr, metadata.kv_indices,
+                metadata.prefix_lens, sm_scale=self.sm_scale,
+                max_len_extend=metadata.max_len_extend,
+                is_cross_attention=is_cross_attention, sliding_window_size=sliding_window_size)
+        assert isinstance(metadata, DecodeMetadata)
+        assert not is_cross_attention and sliding_window_size == 0, (
+            "is_cross_attention / sliding_window_size are only "
+            "supported on the prefill path."
+        )
+        return paged_decode_attention(
+            q, k_cache, v_cache, metadata.kv_indptr, metadata.kv_indices, metadata.num_kv_splits,
+            sm_scale=self.sm_scale, max_kv_splits=metadata.max_kv_splits)
+
+    def store_kv_only(self, k: torch.Tensor, v: torch.Tensor, out_loc: torch.Tensor,
+                      layer_id: int) -> None:
+        """Write K/V without attending (draft calibration, backend.py:174-196)."""
+        self.kvcache.store_kv(k, v, out_loc, layer_id)
+
+    def prepare_metadata(self, batch) -> None:
+        reqs = batch.padded_reqs
+        if batch.is_prefill:
+            batch.attn_metadata = self.build_prefill_metadata(reqs)
+        else:
+            batch.attn_metadata = self.build_decode_metadata(reqs)
+
+    def _gather_indices(self, reqs, kv_lens: Sequence[int]) -> torch.Tensor:
+        return torch.cat([self.page_table[reqs[i].table_idx, : kv_lens[i]]
+                          for i in range(len(reqs))]).to(torch.int32)
+
+    def build_prefill_metadata(self, reqs: List, *, extend_lens: Optional[List[int]] = None,
+                               kv_lens: Optional[List[int]] = None,
+                               positions: Optional[torch.Tensor] = None) -> PrefillMetadata:
+        device = self.page_table.device
+        if extend_lens is None:
+            extend_lens = [req.extend_len for req in reqs]
+        if kv_lens is None:
+            kv_lens = [req.device_len for req in reqs]
+        cached_lens = [kv_lens[i] - extend_lens[i] for i in range(len(reqs))]
+        if positions is None:
+            positions = torch.cat([
+                torch.arange(cached_lens[i], kv_lens[i], dtype=torch.int32, device=device)
+                for i in range(len(reqs))
+            ])
+        return PrefillMetadata(
+            positions=positions,
+            qo_indptr=_build_indptr(extend_lens, device),
+            kv_indptr=_build_indptr(kv_lens, device),
+            kv_indices=self._gather_indices(reqs, kv_lens),
+            prefix_lens=torch.tensor(cached_lens, dtype=torch.int32, device=device),
+            max_len_extend=max(extend_lens),
+        )
+
+    def build_decode_metadata(self, reqs: List, *, kv_lens: Optional[List[int]] = None,
+                              positions: Optional[torch.Tensor] = None) -> DecodeMetadata:
+        device = self.page_table.device
+        if kv_lens is None:
+            kv_lens = [req.device_len for req in reqs]
+        if positions is None:
+            positions = torch.tensor([req.cached_len for req in reqs], dtype=torch.int32,
+                                     device=device)
+        return DecodeMetadata(
+            positions=positions,
+            kv_indptr=_build_indptr(kv_lens, device),
+            kv_indices=self._gather_indices(reqs, kv_lens),
+            num_kv_splits=_compute_num_kv_splits(kv_lens, device),
+            max_kv_splits=MAX_KV_SPLITS,
+        )
+
+
+def _build_indptr(lens: Sequence[int], device=None) -> torch.Tensor:
+    """CSR row pointers ``cumsum([0] + lens)`` as int32 (backend.py:299-301)."""
+    return torch.cumsum(torch.tensor([0] + list(lens), dtype=torch.int32), 0).to(
+        dtype=torch.int32, device=device)
+
+
+def _compute_num_kv_splits(kv_lens: Sequence[int], device=None) -> torch.Tensor:
+    """The reference's split hint ``min(32, max(1, ceil(L / 128)))`` (backend.py:304-307)."""
+    splits = [min(MAX_KV_SPLITS, max(1, (l + 127) // 128)) for l in kv_lens]
+    return torch.tensor(splits, dtype=torch.int32, device=device)

@@ -1,0 +1,262 @@
+"""MI355X counterpart of the reference's ``mini_sglang_mlx_kernel`` module, for the
+paged-attention path only.
+
+Same function names, positional order and keyword names as the nanobind module
+(mini-sglang-mlx-kernel/csrc/bindings.cpp:27-55, mini_sglang_mlx_kernel/__init__.py:1-9);
+``mx.array`` becomes ``torch.Tensor`` on a ROCm device.  Every call is an eager,
+stream-ordered launch of hand-written gfx950 kernels through the C ABI of
+``include/msgl_paged_attention.h``; nothing synchronises with the host and there is no
+other implementation to fall back to.
+
+Argument errors raise ``RuntimeError`` with the reference's message text
+(paged_decode_attention.cpp:25-62, paged_prefill_attention.cpp:31-76,
+store_kv_cache.cpp:22-63).
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from . import _lib
+
+__all__ = ["store_kv_cache", "paged_decode_attention", "paged_prefill_attention"]
+
+_DTYPE_CODE = {torch.bfloat16: _lib.MSGL_DTYPE_BF16, torch.float16: _lib.MSGL_DTYPE_F16}
+
+
+def _fail(op: str, msg: str):
+    raise RuntimeError(f"{op}: {msg}")
+
+
+def _stream_ptr(stream, device) -> int:
+    if stream is None:
+        stream = torch.cuda.current_stream(device)
+    return int(stream.cuda_stream)
+
+
+def _require_device(op: str, *tensors: torch.Tensor) -> torch.device:
+    dev = tensors[0].device
+    if dev.type != "cuda":
+        _fail(op, "tensors must live on a ROCm GPU device (no CPU implementation exists)")
+    for t in tensors:
+        if t.device != dev:
+            _fail(op, "all tensors must be on the same device")
+    return dev
+
+
+def _pool_stride0(op: str, pool: torch.Tensor, name: str) -> int:
+    if pool.stride(2) != 1 or pool.stride(1) != pool.shape[2]:
+        _fail(op, f"{name} must be contiguous in its (num_kv_heads, head_dim) dimensions")
+    # a one-slot pool may report any leading stride
+    return pool.stride(0) if pool.shape[0] > 1 else pool.shape[1] * pool.shape[2]
+
+
+def _int32_1d(op: str, t: torch.Tensor, name: str) -> torch.Tensor:
+    if t.dtype != torch.int32:
+        _fail(op, f"{name} must be int32")
+    return t if t.is_contiguous() else t.contiguous()
+
+
+def _check_rc(op: str, rc: int) -> None:
+    if rc != 0:
+        _fail(op, _lib.strerror(rc))
+
+
+def store_kv_cache(k_cache: torch.Tensor, v_cache: torch.Tensor, indices: torch.Tensor,
+                   k: torch.Tensor, v: torch.Tensor, *, stream=None) -> None:
+    """In place: ``k_cache[indices[r]] = k[r]``, ``v_cache[indices[r]] = v[r]`` (bit copy).
+
+    Drop-in for ``mini_sglang_mlx_kernel.store_kv_cache`` (store_kv_cache.cpp:14-107).
+    ``indices`` must be unique; duplicates race exactly as in the reference.
+    """
+    op = "store_kv_cache"
+    if k_cache.dim() != 3 or v_cache.dim() != 3:
+        _fail(op, "k_cache and v_cache must be 3D (num_pages, num_kv_heads, head_dim)")
+    if indices.dim() != 1:
+        _fail(op, "indices must be 1D")
+    if k.dim() != 3 or v.dim() != 3:
+        _fail(op, "k and v must be 3D (length, num_kv_heads, head_dim)")
+    if not (k_cache.dtype == v_cache.dtype == k.dtype == v.dtype):
+        _fail(op, "k_cache, v_cache, k, v must have the same dtype")
+    if indices.dtype != torch.int32:
+        _fail(op, "indices must be int32")
+    num_pages, num_kv_heads, head_dim = k_cache.shape
+    length = indices.shape[0]
+    if head_dim % 4 != 0:
+        _fail(op, "head_dim must be a multiple of 4")
+    if tuple(v_cache.shape) != (num_pages, num_kv_heads, head_dim):
+        _fail(op, "v_cache shape must match k_cache")
+    if tuple(k.shape) != (length, num_kv_heads, head_dim) or tuple(v.shape) != tuple(k.shape):
+        _fail(op, "k and v shape must be (length, num_kv_heads, head_dim)")
+    if k_cache.element_size() not in (2, 4):
+        _fail(op, "unsupported dtype, must be float16, bfloat16 or float32")
+    dev = _require_device(op, k_cache, v_cache, indices, k, v)
+    if length == 0:
+        return
+    row = num_kv_heads * head_dim
+
+    def _src(t):
+        if t.stride(2) != 1 or t.stride(1) != head_dim:
+            t = t.contiguous()
+        return t, (t.stride(0) if t.shape[0] > 1 else row)
+
+    k, k_stride0 = _src(k)
+    v, v_stride0 = _src(v)
+    indices = indices if indices.is_contiguous() else indices.contiguous()
+    with torch.cuda.device(dev):
+        rc = _lib.load().msgl_store_kv_cache(
+            k_cache.data_ptr(), v_cache.data_ptr(), indices.data_ptr(), k.data_ptr(),
+            v.data_ptr(), length, num_kv_heads, head_dim, num_pages,
+            _pool_stride0(op, k_cache, "k_cache"), _pool_stride0(op, v_cache, "v_cache"),
+            k_stride0, v_stride0, k_cache.element_size(), _stream_ptr(stream, dev))
+    _check_rc(op, rc)
+
+
+def _attention_dtype(op: str, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor) -> int:
+    if q.dtype not in _DTYPE_CODE:
+        _fail(op, "unsupported dtype, must be float16 or bfloat16")
+    if k_cache.dtype != q.dtype or v_cache.dtype != q.dtype:
+        _fail(op, "q, k_cache and v_cache must have the same dtype")
+    if q.dtype != torch.bfloat16:
+        # the reference ships no float16 prefill kernel either
+        # (paged_prefill_attention.metal:646-647); this build is bfloat16 throughout
+        _fail(op, "unsupported dtype, this build provides bfloat16 kernels only")
+    return _DTYPE_CODE[q.dtype]
+
+
+def _workspace(nbytes: int, dev, stream) -> Optional[torch.Tensor]:
+    """Scratch from torch's caching allocator; safe to drop right after the launch because
+    the allocator reuses a block only in stream order (``record_stream`` for a foreign one)."""
+    if nbytes == 0:
+        return None
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    if stream is not None:
+        ws.record_stream(stream)
+    return ws
+
+
+def paged_decode_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                           kv_indptr: torch.Tensor, kv_indices: torch.Tensor,
+                           num_kv_splits: torch.Tensor, sm_scale: float, max_kv_splits: int,
+                           *, stream=None) -> torch.Tensor:
+    """GQA paged decode: ``q (batch, n_q, d)`` against the tokens listed in ``kv_indices``.
+
+    Drop-in for ``mini_sglang_mlx_kernel.paged_decode_attention``
+    (paged_decode_attention.cpp:15-73).  Returns ``(batch, n_q, d)`` in the dtype of ``q``.
+    """
+    op = "paged_decode_attention"
+    if q.dim() != 3:
+        _fail(op, "q must be 3D (batch, num_q_heads, head_dim)")
+    if k_cache.dim() != 3 or v_cache.dim() != 3:
+        _fail(op, "k_cache and v_cache must be 3D (num_pages, num_kv_heads, head_dim)")
+    if kv_indptr.dim() != 1 or kv_indices.dim() != 1 or num_kv_splits.dim() != 1:
+        _fail(op, "kv_indptr, kv_indices, num_kv_splits must be 1D")
+    batch, num_q_heads, head_dim = q.shape
+    num_kv_heads = k_cache.shape[1]
+    if head_dim not in (128, 256):
+        _fail(op, "head_dim must be 128 or 256")
+    if num_q_heads % num_kv_heads != 0:
+        _fail(op, "num_q_heads must be a multiple of num_kv_heads")
+    if num_q_heads // num_kv_heads > 16:
+        _fail(op, "only q_heads/kv_heads <= 16 is supported")
+    if k_cache.shape[2] != head_dim or v_cache.shape[2] != head_dim:
+        _fail(op, "cache head_dim must match q head_dim")
+    if v_cache.shape[1] != num_kv_heads:
+        _fail(op, "v_cache shape must match k_cache")
+    dtype = _attention_dtype(op, q, k_cache, v_cache)
+    kv_indptr = _int32_1d(op, kv_indptr, "kv_indptr")
+    kv_indices = _int32_1d(op, kv_indices, "kv_indices")
+    num_kv_splits = _int32_1d(op, num_kv_splits, "num_kv_splits")
+    if kv_indptr.shape[0] != batch + 1:
+        _fail(op, "kv_indptr must have batch + 1 entries")
+    if num_kv_splits.shape[0] != batch:
+        _fail(op, "num_kv_splits must have batch entries")
+    dev = _require_device(op, q, k_cache, v_cache, kv_indptr, kv_indices, num_kv_splits)
+    q = q if q.is_contiguous() else q.contiguous()
+    out = torch.empty((batch, num_q_heads, head_dim), dtype=q.dtype, device=dev)
+    if batch == 0:
+        return out
+    lib = _lib.load()
+    total_kv = kv_indices.shape[0]
+    with torch.cuda.device(dev):
+        ws_bytes = lib.msgl_paged_decode_workspace_bytes(batch, total_kv, num_q_heads,
+                                                         num_kv_heads, head_dim)
+        ws = _workspace(ws_bytes, dev, stream)
+        rc = lib.msgl_paged_decode_attention(
+            q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), kv_indptr.data_ptr(),
+            kv_indices.data_ptr(), num_kv_splits.data_ptr(), out.data_ptr(),
+            ws.data_ptr() if ws is not None else None, ws_bytes, batch, total_kv, num_q_heads,
+            num_kv_heads, head_dim, k_cache.shape[0], _pool_stride0(op, k_cache, "k_cache"),
+            _pool_stride0(op, v_cache, "v_cache"), float(sm_scale), int(max_kv_splits), dtype,
+            _stream_ptr(stream, dev))
+    _check_rc(op, rc)
+    return out
+
+
+def paged_prefill_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                            qo_indptr: torch.Tensor, kv_indptr: torch.Tensor,
+                            kv_indices: torch.Tensor, prefix_lens: torch.Tensor,
+                            sm_scale: float, max_len_extend: int, *,
+                            is_cross_attention: bool = False, sliding_window_size: int = 0,
+                            stream=None) -> torch.Tensor:
+    """Paged extend attention on top of a cached prefix.
+
+    Drop-in for ``mini_sglang_mlx_kernel.paged_prefill_attention``
+    (paged_prefill_attention.cpp:18-87).  Query ``i`` of request ``b`` sits at position
+    ``prefix_lens[b] + i``; key ``j`` of the request is visible iff
+    ``(is_cross_attention or j <= pos) and (W == 0 or j >= pos - W + 1)``.
+    Returns ``(total_q, n_q, d)`` in the dtype of ``q``; rows of a request beyond
+    ``max_len_extend`` are not computed.
+    """
+    op = "paged_prefill_attention"
+    if q.dim() != 3:
+        _fail(op, "q must be 3D (total_q_tokens, num_q_heads, head_dim)")
+    if k_cache.dim() != 3 or v_cache.dim() != 3:
+        _fail(op, "k_cache and v_cache must be 3D (num_pages, num_kv_heads, head_dim)")
+    if (qo_indptr.dim() != 1 or kv_indptr.dim() != 1 or kv_indices.dim() != 1
+            or prefix_lens.dim() != 1):
+        _fail(op, "qo_indptr, kv_indptr, kv_indices, prefix_lens must be 1D")
+    total_q, num_q_heads, head_dim = q.shape
+    num_kv_heads = k_cache.shape[1]
+    if head_dim not in (128, 256):
+        _fail(op, "head_dim must be 128 or 256")
+    if num_q_heads % num_kv_heads != 0:
+        _fail(op, "num_q_heads must be a multiple of num_kv_heads")
+    if k_cache.shape[2] != head_dim or v_cache.shape[2] != head_dim:
+        _fail(op, "cache head_dim must match q head_dim")
+    if sliding_window_size < 0:
+        _fail(op, "sliding_window_size must be >= 0")
+    batch = qo_indptr.shape[0] - 1
+    if batch <= 0:
+        _fail(op, "batch must be > 0")
+    if v_cache.shape[1] != num_kv_heads:
+        _fail(op, "v_cache shape must match k_cache")
+    dtype = _attention_dtype(op, q, k_cache, v_cache)
+    qo_indptr = _int32_1d(op, qo_indptr, "qo_indptr")
+    kv_indptr = _int32_1d(op, kv_indptr, "kv_indptr")
+    kv_indices = _int32_1d(op, kv_indices, "kv_indices")
+    prefix_lens = _int32_1d(op, prefix_lens, "prefix_lens")
+    if kv_indptr.shape[0] != batch + 1 or prefix_lens.shape[0] != batch:
+        _fail(op, "kv_indptr / prefix_lens length must match qo_indptr")
+    dev = _require_device(op, q, k_cache, v_cache, qo_indptr, kv_indptr, kv_indices, prefix_lens)
+    q = q if q.is_contiguous() else q.contiguous()
+    out = torch.empty((total_q, num_q_heads, head_dim), dtype=q.dtype, device=dev)
+    if total_q == 0:
+        return out
+    lib = _lib.load()
+    total_kv = kv_indices.shape[0]
+    with torch.cuda.device(dev):
+        ws_bytes = lib.msgl_paged_prefill_workspace_bytes(
+            batch, total_q, total_kv, num_q_heads, num_kv_heads, head_dim, int(max_len_extend))
+        ws = _workspace(ws_bytes, dev, stream)
+        rc = lib.msgl_paged_prefill_attention(
+            q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), qo_indptr.data_ptr(),
+            kv_indptr.data_ptr(), kv_indices.data_ptr(), prefix_lens.data_ptr(), out.data_ptr(),
+            ws.data_ptr() if ws is not None else None, ws_bytes, batch, total_q, total_kv,
+            num_q_heads, num_kv_heads, head_dim, k_cache.shape[0],
+            _pool_stride0(op, k_cache, "k_cache"), _pool_stride0(op, v_cache, "v_cache"),
+            float(sm_scale), int(max_len_extend), int(bool(is_cross_attention)),
+            int(sliding_window_size), dtype, _stream_ptr(stream, dev))
+    _check_rc(op, rc)
+    return out

@@ -1,0 +1,79 @@
+"""ctypes binding of ``libmsgl_paged_attention.so`` (the C ABI in ``include/msgl_paged_attention.h``).
+
+The library is built in-tree by ``mini-sglang-mlx_amd/build.py``; nothing here compiles at
+import time and nothing falls back to another implementation: a missing library is an
+``ImportError``-class failure at first use.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+_PKG_ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LIB_PATH = os.path.join(_PKG_ROOT, "lib", "libmsgl_paged_attention.so")
+
+_i64 = ctypes.c_int64
+_i32 = ctypes.c_int32
+_f32 = ctypes.c_float
+_vp = ctypes.c_void_p
+_sz = ctypes.c_size_t
+
+# name -> (restype, argtypes); one entry per MSGL_API declaration of the header
+SIGNATURES = {
+    "msgl_version": (ctypes.c_int, []),
+    "msgl_strerror": (ctypes.c_char_p, [ctypes.c_int]),
+    "msgl_set_tuning": (ctypes.c_int, [_i32, _i64]),
+    "msgl_store_kv_cache": (
+        ctypes.c_int,
+        [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _vp]),
+    "msgl_paged_decode_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64, _i64]),
+    "msgl_paged_decode_attention": (
+        ctypes.c_int,
+        [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i64, _i64, _i64, _i64, _i64, _i64,
+         _i64, _i64, _f32, _i32, _i32, _vp]),
+    "msgl_paged_prefill_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64, _i64, _i64, _i64]),
+    "msgl_paged_prefill_attention": (
+        ctypes.c_int,
+        [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i64, _i64, _i64, _i64, _i64, _i64,
+         _i64, _i64, _i64, _f32, _i32, _i32, _i32, _i32, _vp]),
+}
+
+MSGL_DTYPE_BF16 = 0
+MSGL_DTYPE_F16 = 1
+TUNE_DECODE_CHUNK = 0
+TUNE_SMALLQ_CHUNK = 1
+TUNE_SMALLQ_MAXCOLS = 2
+
+_lib = None
+
+
+class KernelLibraryMissing(ImportError):
+    pass
+
+
+def load() -> ctypes.CDLL:
+    """Load the shared library once; raise loudly if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise KernelLibraryMissing(
+            f"{LIB_PATH} not found: build it with `python mini-sglang-mlx_amd/build.py` "
+            "(or __graft_entry__.build()); there is no fallback implementation")
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (restype, argtypes) in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = restype
+        fn.argtypes = argtypes
+    _lib = lib
+    return lib
+
+
+def strerror(code: int) -> str:
+    return load().msgl_strerror(int(code)).decode()
+
+
+def set_tuning(knob: int, value: int) -> None:
+    rc = load().msgl_set_tuning(int(knob), int(value))
+    if rc != 0:
+        raise ValueError(f"msgl_set_tuning({knob}, {value}): {strerror(rc)}")

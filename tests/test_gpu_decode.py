@@ -1,0 +1,72 @@
+"""Paged GQA decode on the GPU vs the oracle (tolerance: max-abs 2e-2, mean-abs 2e-3)."""
+import pytest
+import torch
+
+from _gpu_util import run_gpu, run_oracle
+from _util import assert_close_bf16
+from mini_sglang_amd.workloads import build_workload
+
+pytestmark = pytest.mark.gpu
+
+
+def _check(wl, gpu, what):
+    print(what, flush=True)
+    got, _ = run_gpu(wl, gpu)
+    want, _ = run_oracle(wl)
+    return assert_close_bf16(got, want, what)
+
+
+@pytest.mark.parametrize("n_q,n_kv", [(8, 8), (16, 8), (32, 8), (64, 8), (16, 1), (6, 3)])
+def test_decode_group_sizes(gpu, n_q, n_kv):
+    wl = build_workload("t", "decode", seed=100 + n_q, n_q=n_q, n_kv=n_kv,
+                        kv_lens=[1, 15, 16, 17, 31, 32, 33, 63, 64, 65, 200, 777], pool_factor=1.3)
+    _check(wl, gpu, f"decode n_q={n_q} n_kv={n_kv}")
+
+
+@pytest.mark.parametrize("chunk", [32, 64, 96, 256, 4096])
+def test_decode_result_independent_of_chunking(gpu, chunk):
+    from mini_sglang_amd_kernel import _lib
+
+    wl = build_workload("t", "decode", seed=7, n_q=32, n_kv=8,
+                        kv_lens=[5, 100, 257, 1000, 2049, 31, 64], pool_factor=1.2)
+    _lib.set_tuning(_lib.TUNE_DECODE_CHUNK, chunk)
+    try:
+        _check(wl, gpu, f"decode chunk={chunk}")
+    finally:
+        _lib.set_tuning(_lib.TUNE_DECODE_CHUNK, 0)
+
+
+def test_decode_empty_request_gives_zeros_and_page_size_one(gpu):
+    wl = build_workload("t", "decode", seed=8, n_q=16, n_kv=8, page_size=1,
+                        kv_lens=[40, 0, 129, 0], pool_factor=2.0)
+    got, _ = run_gpu(wl, gpu)
+    want, _ = run_oracle(wl)
+    assert_close_bf16(got, want, "decode with empty requests")
+    assert torch.count_nonzero(got[1]) == 0 and torch.count_nonzero(got[3]) == 0
+
+
+def test_decode_head_dim_256(gpu):
+    wl = build_workload("t", "decode", seed=9, n_q=8, n_kv=2, head_dim=256,
+                        kv_lens=[3, 64, 130, 515], pool_factor=1.5)
+    _check(wl, gpu, "decode d=256")
+
+
+def test_decode_large_batch_many_requests(gpu):
+    g = torch.Generator().manual_seed(3)
+    lens = torch.randint(1, 300, (150,), generator=g).tolist()
+    wl = build_workload("t", "decode", seed=10, n_q=16, n_kv=4, kv_lens=lens, pool_factor=1.1)
+    _check(wl, gpu, "decode batch=150")
+
+
+def test_decode_strided_pool_views(gpu):
+    """Pools that are planes of a larger (slots, 2, n_kv, d) allocation: stride0 != n_kv*d."""
+    from mini_sglang_amd_kernel import paged_decode_attention
+
+    wl = build_workload("t", "decode", seed=11, n_q=8, n_kv=2, kv_lens=[70, 200], pool_factor=1.0)
+    want, _ = run_oracle(wl)
+    big = torch.stack([wl.k_cache, wl.v_cache], dim=1).to(gpu)  # (slots, 2, n_kv, d)
+    g = wl.to(gpu)
+    out = paged_decode_attention(g.q, big[:, 0], big[:, 1], g.kv_indptr, g.kv_indices,
+                                 g.num_kv_splits, g.sm_scale, g.max_kv_splits)
+    torch.cuda.synchronize()
+    assert_close_bf16(out.cpu(), want, "decode strided pools")

@@ -1,0 +1,160 @@
+"""Paged prefill / extend on the GPU vs the oracle, both routes (MFMA tile kernel for long
+extends, split-K kernel for short query blocks) and all four masks."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from _gpu_util import run_gpu, run_oracle
+from _util import assert_close_bf16
+from mini_sglang_amd.workloads import build_workload
+from test_oracle_known_answers import MASK_CASES, expected_weights, uniform_case
+
+pytestmark = pytest.mark.gpu
+
+MASKS = [(False, 0), (True, 0), (False, 100), (True, 100), (False, 1), (False, 17)]
+
+
+def _check(wl, gpu, what):
+    print(what, flush=True)
+    got, _ = run_gpu(wl, gpu)
+    want, _ = run_oracle(wl)
+    return assert_close_bf16(got, want, what)
+
+
+@pytest.mark.parametrize("q_len,prefix_len,is_cross,window", MASK_CASES)
+def test_reference_mask_cases_closed_form(gpu, q_len, prefix_len, is_cross, window):
+    """The reference's own known-answer cases, run through the GPU operator."""
+    from mini_sglang_amd_kernel import paged_prefill_attention
+
+    d = {k: v.to(gpu) for k, v in uniform_case(q_len, prefix_len).items()}
+    out = paged_prefill_attention(d["q"], d["k_cache"], d["v_cache"], d["qo_indptr"],
+                                  d["kv_indptr"], d["kv_indices"], d["prefix_lens"],
+                                  sm_scale=1.0 / math.sqrt(128), max_len_extend=q_len,
+                                  is_cross_attention=is_cross, sliding_window_size=window)
+    torch.cuda.synchronize()
+    actual = out.float().cpu().numpy()[:, 0, : prefix_len + q_len]
+    np.testing.assert_allclose(actual, expected_weights(q_len, prefix_len, is_cross, window),
+                               rtol=1e-3, atol=1e-3)
+
+
+def test_store_then_prefill_reaches_written_slots(gpu):
+    from mini_sglang_amd_kernel import paged_prefill_attention, store_kv_cache
+
+    q_len = 4
+    page_ids = torch.tensor([3, 1, 4, 2], dtype=torch.int32, device=gpu)
+    q = torch.zeros((q_len, 1, 128), dtype=torch.bfloat16, device=gpu)
+    k = torch.zeros((q_len, 1, 128), dtype=torch.bfloat16, device=gpu)
+    v = torch.zeros((q_len, 1, 128), dtype=torch.float32)
+    for pos in range(q_len):
+        v[pos, 0, pos] = 1.0
+    v = v.to(torch.bfloat16).to(gpu)
+    k_cache = torch.zeros((5, 1, 128), dtype=torch.bfloat16, device=gpu)
+    v_cache = torch.zeros((5, 1, 128), dtype=torch.bfloat16, device=gpu)
+    store_kv_cache(k_cache, v_cache, page_ids, k, v)
+    ip = torch.tensor([0, q_len], dtype=torch.int32, device=gpu)
+    out = paged_prefill_attention(q, k_cache, v_cache, ip, ip, page_ids,
+                                  torch.tensor([0], dtype=torch.int32, device=gpu),
+                                  sm_scale=1.0 / math.sqrt(128), max_len_extend=q_len)
+    torch.cuda.synchronize()
+    np.testing.assert_allclose(out.float().cpu().numpy()[:, 0, :q_len],
+                               expected_weights(q_len, 0, False, 0), rtol=1e-3, atol=1e-3)
+
+
+@pytest.mark.parametrize("is_cross,window", MASKS)
+def test_tile_route_masks(gpu, is_cross, window):
+    # extends long enough for the MFMA tile kernel, ragged, with and without prefix
+    wl = build_workload("t", "prefill", seed=200, n_q=8, n_kv=2,
+                        kv_lens=[70, 300, 64 + 130, 33, 513 + 65],
+                        extend_lens=[70, 100, 130, 33, 65], pool_factor=1.3, store_new=True,
+                        is_cross_attention=is_cross, sliding_window_size=window)
+    _check(wl, gpu, f"tile route cross={is_cross} W={window}")
+
+
+@pytest.mark.parametrize("n_q,n_kv", [(8, 8), (32, 8), (12, 4), (16, 1)])
+def test_tile_route_group_sizes(gpu, n_q, n_kv):
+    wl = build_workload("t", "prefill", seed=210 + n_q, n_q=n_q, n_kv=n_kv,
+                        kv_lens=[200 + 96, 129, 1000 + 257], extend_lens=[96, 129, 257],
+                        pool_factor=1.2, store_new=True)
+    _check(wl, gpu, f"tile route n_q={n_q} n_kv={n_kv}")
+
+
+@pytest.mark.parametrize("is_cross,window", MASKS)
+@pytest.mark.parametrize("q_len", [1, 3, 8])
+def test_splitk_route_masks(gpu, q_len, is_cross, window):
+    # short query blocks (verify / draft proposal): q_len * group <= 64
+    wl = build_workload("t", "prefill", seed=300 + q_len, n_q=16, n_kv=4,
+                        kv_lens=[q_len, 40 + q_len, 333 + q_len, 1500 + q_len],
+                        extend_lens=[q_len] * 4, pool_factor=1.3, store_new=True,
+                        is_cross_attention=is_cross, sliding_window_size=window)
+    _check(wl, gpu, f"split-K route q_len={q_len} cross={is_cross} W={window}")
+
+
+def test_splitk_route_ragged_q_and_chunking(gpu):
+    from mini_sglang_amd_kernel import _lib
+
+    wl = build_workload("t", "prefill", seed=310, n_q=8, n_kv=2,
+                        kv_lens=[5, 100 + 8, 700 + 3, 64 + 16], extend_lens=[5, 8, 3, 16],
+                        pool_factor=1.1, store_new=True, sliding_window_size=50)
+    for chunk in (32, 128, 0):
+        _lib.set_tuning(_lib.TUNE_SMALLQ_CHUNK, chunk)
+        try:
+            _check(wl, gpu, f"split-K route ragged chunk={chunk}")
+        finally:
+            _lib.set_tuning(_lib.TUNE_SMALLQ_CHUNK, 0)
+
+
+def test_both_routes_agree_and_decode_equals_prefill_qlen1(gpu):
+    from mini_sglang_amd_kernel import _lib, paged_decode_attention
+
+    wl = build_workload("t", "prefill", seed=320, n_q=8, n_kv=2, kv_lens=[90 + 8, 8, 400 + 8],
+                        extend_lens=[8, 8, 8], pool_factor=1.0)
+    a, _ = run_gpu(wl, gpu)
+    _lib.set_tuning(_lib.TUNE_SMALLQ_MAXCOLS, -1)  # force the tile kernel
+    try:
+        b, _ = run_gpu(wl, gpu)
+    finally:
+        _lib.set_tuning(_lib.TUNE_SMALLQ_MAXCOLS, 0)
+    want, _ = run_oracle(wl)
+    assert_close_bf16(a, want, "split-K route")
+    assert_close_bf16(b, want, "tile route")
+    # decode(L) == prefill(q_len=1, prefix=L-1)
+    w1 = build_workload("t", "prefill", seed=321, n_q=8, n_kv=2, kv_lens=[77, 1, 300],
+                        extend_lens=[1, 1, 1], pool_factor=1.0)
+    p, g = run_gpu(w1, gpu)
+    splits = torch.ones(3, dtype=torch.int32, device=gpu)
+    dcd = paged_decode_attention(g.q, g.k_cache, g.v_cache, g.kv_indptr, g.kv_indices, splits,
+                                 g.sm_scale, 32)
+    torch.cuda.synchronize()
+    assert_close_bf16(dcd.cpu(), p.float(), "decode vs prefill q_len=1", max_tol=4e-3, mean_tol=2e-4)
+
+
+def test_rows_without_visible_keys_are_zero(gpu):
+    from mini_sglang_amd_kernel import paged_prefill_attention
+
+    wl = build_workload("t", "prefill", seed=330, n_q=4, n_kv=2, kv_lens=[3, 80],
+                        extend_lens=[2, 70], pool_factor=1.0)
+    g = wl.to(gpu)
+    # request 0: kv stream (3 keys) far below the claimed prefix, window 2 => nothing visible
+    prefix = torch.tensor([50, 10], dtype=torch.int32, device=gpu)
+    for max_ext in (70,):
+        out = paged_prefill_attention(g.q, g.k_cache, g.v_cache, g.qo_indptr, g.kv_indptr,
+                                      g.kv_indices, prefix, g.sm_scale, max_ext,
+                                      sliding_window_size=2)
+        torch.cuda.synchronize()
+        assert torch.count_nonzero(out[:2]) == 0
+        assert torch.isfinite(out.float()).all()
+
+
+def test_max_len_extend_smaller_than_a_request_leaves_tail_rows_alone(gpu):
+    from mini_sglang_amd_kernel import paged_prefill_attention
+
+    wl = build_workload("t", "prefill", seed=340, n_q=4, n_kv=2, kv_lens=[20, 30],
+                        extend_lens=[10, 12], pool_factor=1.0)
+    want, _ = run_oracle(wl)
+    g = wl.to(gpu)
+    out = paged_prefill_attention(g.q, g.k_cache, g.v_cache, g.qo_indptr, g.kv_indptr,
+                                  g.kv_indices, g.prefix_lens, g.sm_scale, 12)
+    torch.cuda.synchronize()
+    assert_close_bf16(out.cpu(), want, "reference")
