@@ -1,0 +1,306 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X paged-attention hot path (one GPU).
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--configs 1,2,3,4,5] [--no-check]
+
+A step is one pass of the hot path over one batch of synthetic input that is already
+resident in HBM: the decode operator for the decode shapes, KV-store + extend attention
+for the chunked-prefill shape, the prefill operator for the speculative-verify shape.
+Every step is bracketed by HIP events on the stream the kernels are launched on; the
+median, minimum and mean over the timed steps are reported.
+
+The last line of stdout is ONE JSON object.  Its headline (`value`) is decode-attention
+HBM throughput on shape 2 (Qwen3-8B-shaped paged decode, batch 64); `prefill` carries
+the chunked-prefill TFLOP/s of shape 3 and `all_configs` one row per benchmark shape.
+`roofline.achieved` is ALGORITHMIC bytes (or flops) per step divided by the mean step
+time, which includes the small LSE-merge launch that follows the attention kernel.
+`cpu_baseline` times the CPU oracle (float build, OpenMP) on a bounded sample of the same
+workload on this machine's host cores: a reported baseline, not a target.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "mini-sglang-mlx_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+METRIC = "decode attn HBM TB/s (% of peak) + chunked-prefill attn TFLOP/s (% MFMA peak)"
+HBM_PEAK = 8.0e12
+MFMA_PEAK = 2.5e15
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def time_steps(fn, steps: int, warmup: int):
+    """Per-step durations (ms) from HIP events recorded on torch's current stream, which is
+    the stream every operator launches on."""
+    import torch
+
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    ends = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    t0 = time.perf_counter()
+    for i in range(steps):
+        starts[i].record()
+        fn()
+        ends[i].record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    per = [s.elapsed_time(e) for s, e in zip(starts, ends)]
+    return per, wall_ms
+
+
+def make_step(g):
+    from mini_sglang_amd_kernel import (paged_decode_attention, paged_prefill_attention,
+                                        store_kv_cache)
+
+    if g.kind == "decode":
+        def step():
+            return paged_decode_attention(g.q, g.k_cache, g.v_cache, g.kv_indptr, g.kv_indices,
+                                          g.num_kv_splits, g.sm_scale, g.max_kv_splits)
+    else:
+        def step():
+            if g.out_loc is not None:
+                store_kv_cache(g.k_cache, g.v_cache, g.out_loc, g.new_k, g.new_v)
+            return paged_prefill_attention(
+                g.q, g.k_cache, g.v_cache, g.qo_indptr, g.kv_indptr, g.kv_indices,
+                g.prefix_lens, g.sm_scale, g.max_len_extend,
+                is_cross_attention=g.is_cross_attention,
+                sliding_window_size=g.sliding_window_size)
+    return step
+
+
+def oracle_run(c, precision):
+    import oracle
+
+    if c.out_loc is not None:
+        c = c.clone_pools()
+        oracle.store_kv_cache(c.k_cache, c.v_cache, c.out_loc, c.new_k, c.new_v)
+    if c.kind == "decode":
+        return oracle.paged_decode_attention(
+            c.q, c.k_cache, c.v_cache, c.kv_indptr, c.kv_indices, c.num_kv_splits, c.sm_scale,
+            c.max_kv_splits, precision=precision, return_f32=True)[1], c
+    return oracle.paged_prefill_attention(
+        c.q, c.k_cache, c.v_cache, c.qo_indptr, c.kv_indptr, c.kv_indices, c.prefix_lens,
+        c.sm_scale, c.max_len_extend, is_cross_attention=c.is_cross_attention,
+        sliding_window_size=c.sliding_window_size, precision=precision, return_f32=True)[1], c
+
+
+def sample_requests(wl, max_flops: float):
+    """Requests, shortest first, whose oracle cost stays within ``max_flops`` (at least one)."""
+    from mini_sglang_amd import roofline
+
+    cost = []
+    for b in range(wl.batch):
+        p = wl.kv_lens[b] - wl.extend_lens[b]
+        cost.append((4 * wl.head_dim * wl.n_q * roofline.visible_pairs(
+            p, wl.extend_lens[b], wl.kv_lens[b], wl.is_cross_attention,
+            wl.sliding_window_size), b))
+    cost.sort()
+    picked, total = [], 0.0
+    for c, b in cost:
+        if picked and total + c > max_flops:
+            break
+        picked.append(b)
+        total += c
+    return sorted(picked), total
+
+
+def run_config(cfg: int, variant: str, steps: int, warmup: int, check: bool, cpu_budget_flops: float,
+               dev):
+    import torch
+
+    from mini_sglang_amd.workloads import config_workload
+
+    t0 = time.time()
+    # multi-GiB pools of the long-context shape are drawn on the GPU; the rest on the host
+    wl = config_workload(cfg, variant=variant, pool_device=dev if cfg == 4 else None)
+    g = wl.to(dev)
+    gen_s = time.time() - t0
+    step = make_step(g)
+    out = step()
+    torch.cuda.synchronize()
+    per, wall_ms = time_steps(step, steps, warmup)
+    mean_ms = sum(per) / len(per)
+    med_ms = statistics.median(per)
+    abytes = wl.attention_bytes()
+    aflops = wl.attention_flops()
+    sbytes = wl.store_bytes()
+    bound = "mfma" if (wl.kind == "prefill" and wl.max_len_extend * (wl.n_q // wl.n_kv) > 64) else "hbm"
+    row = {
+        "config": cfg, "workload": wl.name, "kind": wl.kind, "batch": wl.batch,
+        "n_q": wl.n_q, "n_kv": wl.n_kv, "head_dim": wl.head_dim, "page_size": wl.page_size,
+        "total_kv_tokens": int(sum(wl.kv_lens)), "total_q_tokens": int(sum(wl.extend_lens)),
+        "sliding_window": wl.sliding_window_size,
+        "ms_mean": mean_ms, "ms_median": med_ms, "ms_min": min(per),
+        "wall_ms_per_step": wall_ms / steps, "steps": steps, "warmup": warmup,
+        "algorithmic_bytes": abytes, "algorithmic_flops": aflops, "store_bytes": sbytes,
+        "bound": bound, "gen_s": round(gen_s, 1),
+    }
+    if bound == "hbm":
+        row["achieved_TBps"] = abytes / (mean_ms * 1e-3) / 1e12
+        row["roofline_frac"] = row["achieved_TBps"] * 1e12 / HBM_PEAK
+        row["cache_resident"] = abytes < 256e6  # fits the 256 MB Infinity Cache: latency-bound
+    else:
+        row["achieved_TFLOPs"] = aflops / (mean_ms * 1e-3) / 1e12
+        row["roofline_frac"] = row["achieved_TFLOPs"] * 1e12 / MFMA_PEAK
+
+    if check or cpu_budget_flops > 0:
+        import oracle  # noqa: F401  (checker and CPU baseline only)
+
+        reqs, flops = sample_requests(wl, max(cpu_budget_flops, 2e10))
+        sub = wl.select(reqs).to("cpu")
+        torch.set_num_threads(os.cpu_count() or 1)
+        t1 = time.perf_counter()
+        want, ref = oracle_run(sub, "f32")
+        cpu_s = time.perf_counter() - t1
+        if check:
+            gsub = sub.to(dev)
+            got = make_step(gsub)()
+            torch.cuda.synchronize()
+            diff = (got.float().cpu() - want).abs()
+            row["max_abs_err"] = float(diff.max())
+            row["mean_abs_err"] = float(diff.mean())
+            row["checked_requests"] = len(reqs)
+            row["parity_ok"] = bool(row["max_abs_err"] <= 2e-2 and row["mean_abs_err"] <= 2e-3)
+            if sub.out_loc is not None:
+                row["kv_pool_bit_exact"] = bool(
+                    torch.equal(gsub.k_cache.cpu().view(torch.int16), ref.k_cache.view(torch.int16))
+                    and torch.equal(gsub.v_cache.cpu().view(torch.int16), ref.v_cache.view(torch.int16)))
+        threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+        cpu = {"seconds": cpu_s, "cores": threads, "kind": "port",
+               "sample": f"{len(reqs)} of {wl.batch} requests (shortest first), CPU oracle float "
+                         f"build with OpenMP, one pass, MLX not installed"}
+        if bound == "hbm":
+            cpu["value"] = sub.attention_bytes() / cpu_s / 1e12
+            cpu["unit"] = "TB/s"
+        else:
+            cpu["value"] = sub.attention_flops() / cpu_s / 1e12
+            cpu["unit"] = "TFLOP/s"
+        row["cpu_baseline"] = cpu
+    del g, out
+    torch.cuda.empty_cache()
+    return row
+
+
+def load_traffic():
+    """Measured HBM bytes per launch from the committed rocprofv3 counter summaries."""
+    path = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    if os.path.exists(path):
+        with open(path) as f:
+            return json.load(f)
+    return {}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--configs", default="2,3,1,5,5w,4")
+    ap.add_argument("--no-check", action="store_true", help="skip the oracle comparison")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--tune", action="append", default=[], metavar="KNOB=VALUE",
+                    help="set a msgl_set_tuning knob (benchmarking only), e.g. 0=512")
+    ap.add_argument("--cpu-flops", type=float, default=3e11,
+                    help="flop budget of the CPU baseline sample per shape")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs the hot path on ONE GPU; --gpus N with N > 1 is "
+                 "not supported (no collective or sharding code is part of it)")
+
+    import torch
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no ROCm GPU visible")
+    from mini_sglang_amd_kernel import _lib
+
+    _lib.load()  # fail loudly if the HIP library was not built
+    for kv in args.tune:
+        knob, value = kv.split("=")
+        _lib.set_tuning(int(knob), int(value))
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    traffic = load_traffic()
+
+    rows = []
+    for tok in [t.strip() for t in args.configs.split(",") if t.strip()]:
+        cfg, variant = (int(tok[:-1]), "window") if tok.endswith("w") else (int(tok), "")
+        steps = args.steps if cfg != 4 else max(5, args.steps // 5)
+        budget = 0.0 if args.no_cpu_baseline else args.cpu_flops
+        row = run_config(cfg, variant, steps, args.warmup if cfg != 4 else max(2, args.warmup // 3),
+                         not args.no_check, budget, dev)
+        rows.append(row)
+        perf = (f"{row['achieved_TBps']:.3f} TB/s" if row["bound"] == "hbm"
+                else f"{row['achieved_TFLOPs']:.1f} TFLOP/s")
+        log(f"[cfg {tok}] {row['workload']}: {row['ms_mean']*1e3:.1f} us mean "
+            f"({row['ms_min']*1e3:.1f} min)  {perf}  {row['roofline_frac']*100:.1f}% of "
+            f"{row['bound']} peak  err max {row.get('max_abs_err', float('nan')):.2e} "
+            f"mean {row.get('mean_abs_err', float('nan')):.2e}  cpu "
+            f"{row.get('cpu_baseline', {}).get('value', float('nan')):.4f} "
+            f"{row.get('cpu_baseline', {}).get('unit', '')}")
+
+    def find(cfg, variant_window=False):
+        for r in rows:
+            if r["config"] == cfg and (r["sliding_window"] > 0) == variant_window:
+                return r
+        return None
+
+    head = find(2) or next((r for r in rows if r["bound"] == "hbm"), rows[0])
+    pre = find(3)
+
+    def roofline_obj(r):
+        if r["bound"] == "hbm":
+            return {"bound": "hbm", "achieved": r["achieved_TBps"] * 1e3, "peak": HBM_PEAK / 1e9,
+                    "unit": "GB/s", "frac": r["roofline_frac"],
+                    "traffic": traffic.get(r["workload"])}
+        return {"bound": "mfma", "achieved": r["achieved_TFLOPs"], "peak": MFMA_PEAK / 1e12,
+                "unit": "TFLOP/s", "frac": r["roofline_frac"], "traffic": traffic.get(r["workload"])}
+
+    def cpu_obj(r):
+        c = r.get("cpu_baseline")
+        if not c:
+            return None
+        return {"value": c["value"], "unit": c["unit"], "cores": c["cores"], "kind": c["kind"],
+                "sample": c["sample"]}
+
+    result = {
+        "metric": METRIC,
+        "value": head.get("achieved_TBps", head.get("achieved_TFLOPs")),
+        "unit": "TB/s" if head["bound"] == "hbm" else "TFLOP/s",
+        "n_gpus": 1, "steps": head["steps"], "warmup": head["warmup"],
+        "ms_per_step": head["ms_mean"], "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"{head['workload']}: paged GQA decode, batch {head['batch']}, "
+                               f"{head['n_q']} q / {head['n_kv']} kv heads, head_dim "
+                               f"{head['head_dim']}, page size {head['page_size']}, "
+                               f"{head['total_kv_tokens']} kv tokens, bf16 pool",
+                   "parallelism": "1 GPU"},
+        "roofline": roofline_obj(head),
+        "cpu_baseline": cpu_obj(head),
+    }
+    if pre is not None:
+        result["prefill"] = {
+            "workload": f"{pre['workload']}: 8 requests x 512-token causal extend on cached "
+                        f"prefixes, {pre['n_q']} q / {pre['n_kv']} kv heads, KV-store included",
+            "value": pre["achieved_TFLOPs"], "unit": "TFLOP/s", "ms_per_step": pre["ms_mean"],
+            "roofline": roofline_obj(pre), "cpu_baseline": cpu_obj(pre),
+            "parity_ok": pre.get("parity_ok"), "kv_pool_bit_exact": pre.get("kv_pool_bit_exact"),
+        }
+    result["all_configs"] = rows
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

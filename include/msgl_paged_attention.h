@@ -150,10 +150,12 @@ MSGL_API int msgl_paged_prefill_attention(const void* q, const void* k_cache, co
  *   MSGL_TUNE_DECODE_CHUNK   tokens per split-K work item in decode (multiple of 32)
  *   MSGL_TUNE_SMALLQ_CHUNK   same for the short-query route of prefill
  *   MSGL_TUNE_SMALLQ_MAXCOLS largest q_len*group routed to the split-K kernel
+ *   MSGL_TUNE_PREFILL_VARIANT tiling of the MFMA kernel (0: 8 waves x 32 rows, 1: 4 x 64)
  */
 #define MSGL_TUNE_DECODE_CHUNK 0
 #define MSGL_TUNE_SMALLQ_CHUNK 1
 #define MSGL_TUNE_SMALLQ_MAXCOLS 2
+#define MSGL_TUNE_PREFILL_VARIANT 3
 MSGL_API int msgl_set_tuning(int32_t knob, int64_t value);
 
 #ifdef __cplusplus

@@ -58,6 +58,10 @@ struct PrefillArgs {
   int32_t is_cross, window;
 };
 int launch_prefill_tile(const PrefillArgs& a, hipStream_t stream);
+// benchmarking switch between the two tilings of the MFMA kernel (0: 8 waves x 32 rows,
+// 1: 4 waves x 64 rows); both cover 256 rows per workgroup
+int tile_variant();
+void set_tile_variant(int v);
 
 inline int check_launch() { return hipGetLastError() == hipSuccess ? MSGL_OK : MSGL_ERR_LAUNCH; }
 

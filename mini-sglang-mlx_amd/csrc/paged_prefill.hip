@@ -22,6 +22,8 @@
 //   waves skip tiles none of their rows can see.
 //
 // Algorithmic flops: 4 * D per visible (query, key) pair and q head (QK^T + PV).
+#include <atomic>
+
 #include "msgl_device.h"
 #include "msgl_internal.h"
 
@@ -44,13 +46,12 @@ struct PrefillParams {
   float scale_log2e;
 };
 
-constexpr int kRows = 256;  // rows per workgroup
-constexpr int kBN = 64;     // keys per tile
+constexpr int kBN = 64;  // keys per tile
 // A stale row max is kept until the new one exceeds it by this much (base-2 exponent):
 // P stays below 2^kLazy, far inside bf16 / fp32 range, and O is rescaled rarely.
 constexpr float kLazy = 8.0f;
 
-template <int D>
+template <int D, int ROWS>
 struct Smem {
   static constexpr int KROW = D + 8;    // bf16 elements per K row (16 B pad)
   static constexpr int VROW = kBN + 8;  // bf16 elements per V^T row
@@ -58,14 +59,18 @@ struct Smem {
   static constexpr int V_BYTES = D * VROW * 2;
   static constexpr int STAGE_BYTES = K_BYTES + V_BYTES;
   static constexpr int OROW = D + 8;
-  static constexpr int O_BYTES = kRows * OROW * 2;
+  static constexpr int O_BYTES = ROWS * OROW * 2;
   static constexpr int TOTAL = (2 * STAGE_BYTES > O_BYTES) ? 2 * STAGE_BYTES : O_BYTES;
 };
 
-template <int D>
-__global__ __launch_bounds__(256) void prefill_tile_kernel(PrefillParams p) {
+// RT = 32-row tiles per wave, NW = waves per workgroup; the workgroup covers NW*RT*32 rows.
+template <int D, int RT, int NW>
+__global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) {
   static_assert(D == 128, "tile kernel is instantiated for head_dim 128");
-  using S = Smem<D>;
+  constexpr int kRows = NW * RT * 32;
+  constexpr int KPT = kBN * 16 / (NW * 64);  // keys staged per thread (16 threads per row)
+  static_assert(KPT == 4 || KPT == 2, "staging assumes 256 or 512 threads");
+  using S = Smem<D, kRows>;
   constexpr int KSTEPS = D / 16;  // k-steps of QK^T
   constexpr int DT = D / 32;      // 32-row tiles of O^T
   __shared__ __attribute__((aligned(16))) unsigned char smem[S::TOTAL];
@@ -105,18 +110,16 @@ __global__ __launch_bounds__(256) void prefill_tile_kernel(PrefillParams p) {
   const int n_tiles = (k_hi - k_lo + kBN - 1) / kBN;
 
   // ---- per-lane rows: Q operand, visibility bounds ---------------------------------
-  bf16x8_t qreg[2][KSTEPS];
-  int row_lo[2], row_hi[2];
-  int64_t out_off[2];
+  bf16x8_t qreg[RT][KSTEPS];
+  int row_lo[RT], row_hi[RT];
   int w_lo_min = 0x7fffffff, w_lo_max = -0x7fffffff, w_hi_min = 0x7fffffff, w_hi_max = -1;
 #pragma unroll
-  for (int rt = 0; rt < 2; ++rt) {
-    const int row = row0 + w * 64 + rt * 32 + c32;
+  for (int rt = 0; rt < RT; ++rt) {
+    const int row = row0 + (w * RT + rt) * 32 + c32;
     const bool valid = row < rows_total;
     const int qi = valid ? row / p.group : 0;
     const int hh = valid ? row - qi * p.group : 0;
     const int64_t off = ((int64_t)(q_start + qi) * p.n_q + kvh * p.group + hh) * D;
-    out_off[rt] = off;
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) {
       u32x4_t raw = {0u, 0u, 0u, 0u};
@@ -150,28 +153,33 @@ __global__ __launch_bounds__(256) void prefill_tile_kernel(PrefillParams p) {
   w_hi_min = __builtin_amdgcn_readfirstlane(w_hi_min);
   w_hi_max = __builtin_amdgcn_readfirstlane(w_hi_max);
 
-  f32x16_t oacc[DT][2];
+  f32x16_t oacc[DT][RT];
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-    for (int rt = 0; rt < 2; ++rt)
+    for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
       for (int i = 0; i < 16; ++i) oacc[dt][rt][i] = 0.f;
-  float m_run[2] = {kNegInf, kNegInf};
-  float l_run[2] = {0.f, 0.f};
+  float m_run[RT], l_run[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    m_run[rt] = kNegInf;
+    l_run[rt] = 0.f;
+  }
 
-  // ---- staging: thread (kg, c) moves keys 4kg..4kg+3, dims 8c..8c+7 ------------------
+  // ---- staging: thread (kg, c) moves keys KPT*kg .. KPT*kg+KPT-1, dims 8c..8c+7 -------
   const int kg = tid >> 4;
   const int c = tid & 15;
-  const int kgs = (kg & ~3) | ((kg & 1) << 1) | ((kg >> 1) & 1);  // key bits 2 and 3 swapped
+  const int key0 = kg * KPT;
+  const int pos0 = (key0 & ~12) | ((key0 & 4) << 1) | ((key0 & 8) >> 1);  // key bits 2 <-> 3
   const int32_t* idx_base = p.kv_indices + kv_start;
   const uint16_t* kbase = p.k_cache + (int64_t)kvh * D + c * 8;
   const uint16_t* vbase = p.v_cache + (int64_t)kvh * D + c * 8;
-  u32x4_t kr[4], vr[4];
+  u32x4_t kr[KPT], vr[KPT];
   auto stage_load = [&](int tb) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int64_t slot = idx_base[min(tb + 4 * kg + i, kn - 1)];
+    for (int i = 0; i < KPT; ++i) {
+      const int64_t slot = idx_base[min(tb + key0 + i, kn - 1)];
       kr[i] = ld_global_b128(kbase + slot * p.k_stride0);
       vr[i] = ld_global_b128(vbase + slot * p.v_stride0);
     }
@@ -180,15 +188,23 @@ __global__ __launch_bounds__(256) void prefill_tile_kernel(PrefillParams p) {
     unsigned char* ks = smem + buf * S::STAGE_BYTES;
     unsigned char* vs = ks + S::K_BYTES;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-      *reinterpret_cast<u32x4_t*>(ks + ((4 * kg + i) * S::KROW + c * 8) * 2) = kr[i];
+    for (int i = 0; i < KPT; ++i)
+      *reinterpret_cast<u32x4_t*>(ks + ((key0 + i) * S::KROW + c * 8) * 2) = kr[i];
     // V^T row of dim 8c+n is 16n+c: the 16 lanes of one write hit consecutive rows
 #pragma unroll
     for (int n = 0; n < 8; ++n) {
-      u32x2_t t;
-      t[0] = (n & 1) ? pack_hi16(vr[0][n >> 1], vr[1][n >> 1]) : pack_lo16(vr[0][n >> 1], vr[1][n >> 1]);
-      t[1] = (n & 1) ? pack_hi16(vr[2][n >> 1], vr[3][n >> 1]) : pack_lo16(vr[2][n >> 1], vr[3][n >> 1]);
-      *reinterpret_cast<u32x2_t*>(vs + ((16 * n + c) * S::VROW + 4 * kgs) * 2) = t;
+      unsigned char* dst = vs + ((16 * n + c) * S::VROW + pos0) * 2;
+      const uint32_t t0 = (n & 1) ? pack_hi16(vr[0][n >> 1], vr[1][n >> 1])
+                                  : pack_lo16(vr[0][n >> 1], vr[1][n >> 1]);
+      if constexpr (KPT == 4) {
+        u32x2_t t;
+        t[0] = t0;
+        t[1] = (n & 1) ? pack_hi16(vr[2][n >> 1], vr[3][n >> 1])
+                       : pack_lo16(vr[2][n >> 1], vr[3][n >> 1]);
+        *reinterpret_cast<u32x2_t*>(dst) = t;
+      } else {
+        *reinterpret_cast<uint32_t*>(dst) = t0;
+      }
     }
   };
 
@@ -196,11 +212,11 @@ __global__ __launch_bounds__(256) void prefill_tile_kernel(PrefillParams p) {
     const unsigned char* ks = smem + buf * S::STAGE_BYTES;
     const unsigned char* vs = ks + S::K_BYTES;
     // S^T[key][row]: lane holds key = tb + 32kt + 8(i/4) + 4h + i%4, row = 32rt + c32
-    f32x16_t s[2][2];
+    f32x16_t s[2][RT];
 #pragma unroll
     for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-      for (int rt = 0; rt < 2; ++rt)
+      for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
         for (int i = 0; i < 16; ++i) s[kt][rt][i] = 0.f;
 #pragma unroll
@@ -209,14 +225,14 @@ __global__ __launch_bounds__(256) void prefill_tile_kernel(PrefillParams p) {
       for (int kt = 0; kt < 2; ++kt) {
         const bf16x8_t a = as_bf16x8(*reinterpret_cast<const u32x4_t*>(
             ks + ((kt * 32 + c32) * S::KROW + kstep * 16 + h * 8) * 2));
-        s[kt][0] = mfma_32x32x16(a, qreg[0][kstep], s[kt][0]);
-        s[kt][1] = mfma_32x32x16(a, qreg[1][kstep], s[kt][1]);
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) s[kt][rt] = mfma_32x32x16(a, qreg[rt][kstep], s[kt][rt]);
       }
 
     const bool need_mask = (tb < w_lo_max) || (tb + kBN - 1 > w_hi_min);
-    bf16x8_t pb[2][4];
+    bf16x8_t pb[RT][4];
 #pragma unroll
-    for (int rt = 0; rt < 2; ++rt) {
+    for (int rt = 0; rt < RT; ++rt) {
       if (need_mask) {
 #pragma unroll
         for (int kt = 0; kt < 2; ++kt)
@@ -283,8 +299,8 @@ __global__ __launch_bounds__(256) void prefill_tile_kernel(PrefillParams p) {
       for (int dt = 0; dt < DT; ++dt) {
         const bf16x8_t a = as_bf16x8(*reinterpret_cast<const u32x4_t*>(
             vs + ((dt * 32 + c32) * S::VROW + 16 * u + 8 * h) * 2));
-        oacc[dt][0] = mfma_32x32x16(a, pb[0][u], oacc[dt][0]);
-        oacc[dt][1] = mfma_32x32x16(a, pb[1][u], oacc[dt][1]);
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) oacc[dt][rt] = mfma_32x32x16(a, pb[rt][u], oacc[dt][rt]);
       }
   };
 
@@ -309,11 +325,11 @@ __global__ __launch_bounds__(256) void prefill_tile_kernel(PrefillParams p) {
   // X = 8((i/4)&1) + 4h + i%4.
   unsigned char* os = smem;
 #pragma unroll
-  for (int rt = 0; rt < 2; ++rt) {
+  for (int rt = 0; rt < RT; ++rt) {
     float l = l_run[rt];
     l += __shfl_xor(l, 32, kWave);
     const float inv = (l > 0.f) ? 1.0f / l : 0.f;
-    const int lrow = w * 64 + rt * 32 + c32;
+    const int lrow = (w * RT + rt) * 32 + c32;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       u32x4_t wv;
@@ -325,9 +341,10 @@ __global__ __launch_bounds__(256) void prefill_tile_kernel(PrefillParams p) {
     }
   }
   __syncthreads();
+  constexpr int ROWS_PER_PASS = NW * 4;
 #pragma unroll 4
-  for (int pass = 0; pass < kRows / 16; ++pass) {
-    const int lrow = pass * 16 + (tid >> 4);
+  for (int pass = 0; pass < kRows / ROWS_PER_PASS; ++pass) {
+    const int lrow = pass * ROWS_PER_PASS + (tid >> 4);
     const int row = row0 + lrow;
     if (row < rows_total) {
       const int qi = row / p.group;
@@ -336,10 +353,13 @@ __global__ __launch_bounds__(256) void prefill_tile_kernel(PrefillParams p) {
       st_global_b128(p.out + ((int64_t)(q_start + qi) * p.n_q + kvh * p.group + hh) * D + c * 8, v);
     }
   }
-  (void)out_off;
 }
 
 }  // namespace
+
+static std::atomic<int> g_tile_variant{0};
+int tile_variant() { return g_tile_variant.load(); }
+void set_tile_variant(int v) { g_tile_variant.store(v); }
 
 int launch_prefill_tile(const PrefillArgs& a, hipStream_t stream) {
   if (a.head_dim != 128) return MSGL_ERR_HEAD_DIM;
@@ -362,15 +382,22 @@ int launch_prefill_tile(const PrefillArgs& a, hipStream_t stream) {
   p.is_cross = a.is_cross;
   p.window = a.window;
   p.scale_log2e = a.sm_scale * kLog2e;
+  const int variant = tile_variant();
+  const int64_t block_rows = 256;
   const int64_t rows = (int64_t)a.max_len_extend * p.group;
-  const int64_t n_qblk = (rows + kRows - 1) / kRows;
+  const int64_t n_qblk = (rows + block_rows - 1) / block_rows;
   const int64_t n_pairs = a.batch * a.n_kv;
   const int64_t n_blocks = (n_pairs + 7) / 8 * 8 * n_qblk;
   if (n_qblk <= 0 || n_blocks <= 0) return MSGL_OK;
   if (n_blocks > 0x7fffffffLL) return MSGL_ERR_SHAPE;
   p.n_qblk = (int32_t)n_qblk;
   p.n_pairs = (int32_t)n_pairs;
-  hipLaunchKernelGGL((prefill_tile_kernel<128>), dim3((unsigned)n_blocks), dim3(256), 0, stream, p);
+  if (variant == 1)
+    hipLaunchKernelGGL((prefill_tile_kernel<128, 2, 4>), dim3((unsigned)n_blocks), dim3(256), 0,
+                       stream, p);
+  else
+    hipLaunchKernelGGL((prefill_tile_kernel<128, 1, 8>), dim3((unsigned)n_blocks), dim3(512), 0,
+                       stream, p);
   return check_launch();
 }
 

@@ -113,14 +113,25 @@ def _indptr(lens) -> torch.Tensor:
     return torch.cumsum(torch.tensor([0] + list(lens), dtype=torch.int64), 0).to(torch.int32)
 
 
-def _randn_bf16(shape, g: torch.Generator) -> torch.Tensor:
-    """fp32 N(0,1) rounded to bf16, drawn in slabs so the fp32 temporary stays small."""
-    out = torch.empty(shape, dtype=torch.bfloat16)
+def _randn_bf16(shape, g: torch.Generator, device=None) -> torch.Tensor:
+    """fp32 N(0,1) rounded to bf16, drawn in slabs so the fp32 temporary stays small.
+
+    With a non-CPU ``device`` the values are drawn there, from a generator seeded by the next
+    draw of ``g`` (multi-GiB pools take a minute on host cores); the stream of values then
+    differs from the CPU one but is still a function of the seed alone.
+    """
+    device = torch.device(device) if device is not None else torch.device("cpu")
+    gen = g
+    if device.type != "cpu":
+        gen = torch.Generator(device=device)
+        gen.manual_seed(int(torch.randint(0, 2**31 - 1, (1,), generator=g)))
+    out = torch.empty(shape, dtype=torch.bfloat16, device=device)
     flat = out.view(-1)
     step = 1 << 26
     for s in range(0, flat.numel(), step):
         n = min(step, flat.numel() - s)
-        flat[s:s + n] = torch.randn(n, generator=g, dtype=torch.float32).to(torch.bfloat16)
+        flat[s:s + n] = torch.randn(n, generator=gen, dtype=torch.float32,
+                                    device=device).to(torch.bfloat16)
     return out
 
 
@@ -134,7 +145,8 @@ def build_workload(name: str, kind: str, *, seed: int, n_q: int, n_kv: int, head
                    pool_pages: Optional[int] = None, pool_factor: float = 1.0,
                    store_new: bool = False, is_cross_attention: bool = False,
                    sliding_window_size: int = 0,
-                   generator: Optional[torch.Generator] = None) -> PagedWorkload:
+                   generator: Optional[torch.Generator] = None,
+                   pool_device=None) -> PagedWorkload:
     g = generator if generator is not None else torch.Generator().manual_seed(seed)
     batch = len(kv_lens)
     if extend_lens is None:
@@ -155,8 +167,8 @@ def build_workload(name: str, kind: str, *, seed: int, n_q: int, n_kv: int, head
     kv_indices = (torch.cat(pieces) if pieces else torch.zeros(0, dtype=torch.int64)).to(torch.int32)
     kv_indptr = _indptr(kv_lens)
     num_slots = pool_pages * page_size
-    k_cache = _randn_bf16((num_slots, n_kv, head_dim), g)
-    v_cache = _randn_bf16((num_slots, n_kv, head_dim), g)
+    k_cache = _randn_bf16((num_slots, n_kv, head_dim), g, pool_device)
+    v_cache = _randn_bf16((num_slots, n_kv, head_dim), g, pool_device)
     total_q = sum(extend_lens)
     q = _randn_bf16((total_q, n_q, head_dim), g)
     wl = PagedWorkload(
@@ -189,29 +201,30 @@ def _scaled(x: int, scale: float, floor: int = 1) -> int:
     return max(floor, int(round(x * scale)))
 
 
-def config_workload(cfg: int, *, scale: float = 1.0, variant: str = "") -> PagedWorkload:
+def config_workload(cfg: int, *, scale: float = 1.0, variant: str = "",
+                    pool_device=None) -> PagedWorkload:
     """Workload of benchmark shape ``cfg`` (1..5); ``scale`` < 1 shrinks the lengths (and, for
     shape 3, the extend) for CPU-sized tests.  ``variant="window"`` selects the sliding
-    window 1024 run of shape 5."""
+    window 1024 run of shape 5.  ``pool_device`` draws the two pools on that device."""
     g = torch.Generator().manual_seed(SEED_BASE + cfg)
     if cfg == 1:
         lens = [_scaled(l, scale) for l in (37, 128, 500, 1023)]
         return build_workload("cfg1_decode_qwen3_0.6b", "decode", seed=0, generator=g, n_q=16,
-                              n_kv=8, kv_lens=lens, pool_pages=512)
+                              n_kv=8, kv_lens=lens, pool_pages=512, pool_device=pool_device)
     if cfg == 2:
         lens = _randint_list(_scaled(1024, scale), _scaled(8192, scale), 64, g)
         return build_workload("cfg2_decode_qwen3_8b", "decode", seed=0, generator=g, n_q=32,
-                              n_kv=8, kv_lens=lens, pool_factor=1.5)
+                              n_kv=8, kv_lens=lens, pool_factor=1.5, pool_device=pool_device)
     if cfg == 3:
         ext = _scaled(512, scale)
         prefixes = _randint_list(0, _scaled(16384, scale), 8, g)
         return build_workload("cfg3_extend_qwen3_8b", "prefill", seed=0, generator=g, n_q=32,
                               n_kv=8, kv_lens=[p + ext for p in prefixes], extend_lens=[ext] * 8,
-                              pool_factor=1.5, store_new=True)
+                              pool_factor=1.5, store_new=True, pool_device=pool_device)
     if cfg == 4:
         lens = _randint_list(_scaled(32768, scale), _scaled(131072, scale), 16, g)
         return build_workload("cfg4_decode_qwen3_32b_long", "decode", seed=0, generator=g, n_q=64,
-                              n_kv=8, kv_lens=lens, pool_factor=1.0)
+                              n_kv=8, kv_lens=lens, pool_factor=1.0, pool_device=pool_device)
     if cfg == 5:
         prefixes = _randint_list(_scaled(2048, scale), _scaled(8192, scale), 32, g)
         window = 0
@@ -221,5 +234,6 @@ def config_workload(cfg: int, *, scale: float = 1.0, variant: str = "") -> Paged
             name = "cfg5_verify_window"
         return build_workload(name, "prefill", seed=0, generator=g, n_q=32, n_kv=8,
                               kv_lens=[p + 8 for p in prefixes], extend_lens=[8] * 32,
-                              pool_factor=1.0, sliding_window_size=window)
+                              pool_factor=1.0, sliding_window_size=window,
+                              pool_device=pool_device)
     raise ValueError(f"unknown benchmark shape {cfg}")

@@ -43,6 +43,7 @@ MSGL_DTYPE_F16 = 1
 TUNE_DECODE_CHUNK = 0
 TUNE_SMALLQ_CHUNK = 1
 TUNE_SMALLQ_MAXCOLS = 2
+TUNE_PREFILL_VARIANT = 3
 
 _lib = None
 

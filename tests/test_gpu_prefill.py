@@ -62,18 +62,28 @@ def test_store_then_prefill_reaches_written_slots(gpu):
                                expected_weights(q_len, 0, False, 0), rtol=1e-3, atol=1e-3)
 
 
+@pytest.fixture(params=[0, 1], ids=["8x32rows", "4x64rows"])
+def tile_variant(request):
+    """Both tilings of the MFMA kernel are product code; each is checked."""
+    from mini_sglang_amd_kernel import _lib
+
+    _lib.set_tuning(_lib.TUNE_PREFILL_VARIANT, request.param)
+    yield request.param
+    _lib.set_tuning(_lib.TUNE_PREFILL_VARIANT, 0)
+
+
 @pytest.mark.parametrize("is_cross,window", MASKS)
-def test_tile_route_masks(gpu, is_cross, window):
+def test_tile_route_masks(gpu, tile_variant, is_cross, window):
     # extends long enough for the MFMA tile kernel, ragged, with and without prefix
     wl = build_workload("t", "prefill", seed=200, n_q=8, n_kv=2,
                         kv_lens=[70, 300, 64 + 130, 33, 513 + 65],
                         extend_lens=[70, 100, 130, 33, 65], pool_factor=1.3, store_new=True,
                         is_cross_attention=is_cross, sliding_window_size=window)
-    _check(wl, gpu, f"tile route cross={is_cross} W={window}")
+    _check(wl, gpu, f"tile route variant={tile_variant} cross={is_cross} W={window}")
 
 
 @pytest.mark.parametrize("n_q,n_kv", [(8, 8), (32, 8), (12, 4), (16, 1)])
-def test_tile_route_group_sizes(gpu, n_q, n_kv):
+def test_tile_route_group_sizes(gpu, tile_variant, n_q, n_kv):
     wl = build_workload("t", "prefill", seed=210 + n_q, n_q=n_q, n_kv=n_kv,
                         kv_lens=[200 + 96, 129, 1000 + 257], extend_lens=[96, 129, 257],
                         pool_factor=1.2, store_new=True)
