@@ -94,8 +94,8 @@ MSGL_API size_t msgl_paged_decode_workspace_bytes(int64_t batch, int64_t total_k
  *   q   (batch, num_q_heads, head_dim)      out (batch, num_q_heads, head_dim)
  *   kv_indptr (batch+1)   kv_indices (total_kv)   num_kv_splits (batch)
  * Request b attends to all kv_indptr[b+1]-kv_indptr[b] tokens listed for it.
- * The KV range of a request is cut into fixed-size chunks chosen for MI355X
- * occupancy; partial results are merged by log-sum-exp.  The result does not
+ * The concatenated KV stream of the batch is cut into equal segments, one resident round of
+ * workgroups on MI355X; partial results are merged by log-sum-exp.  The result does not
  * depend on the split, so `num_kv_splits` / `max_kv_splits` (the reference's
  * split hints, backend.py:304-307) are accepted and validated but do not steer
  * the cut.  A request with no tokens gets zeros (the reference leaves its rows
@@ -147,13 +147,13 @@ MSGL_API int msgl_paged_prefill_attention(const void* q, const void* k_cache, co
 /*
  * Tuning knobs, for benchmarking only (0 = built-in heuristic).  Process-wide,
  * read at launch time; not part of the reference surface.
- *   MSGL_TUNE_DECODE_CHUNK   tokens per split-K work item in decode (multiple of 32)
- *   MSGL_TUNE_SMALLQ_CHUNK   same for the short-query route of prefill
+ *   MSGL_TUNE_SEGMENTS       segments the split-K kernel cuts the visible token stream into
+ *   MSGL_TUNE_MIN_SEGMENT    smallest segment length in tokens (multiple of 64)
  *   MSGL_TUNE_SMALLQ_MAXCOLS largest q_len*group routed to the split-K kernel
  *   MSGL_TUNE_PREFILL_VARIANT tiling of the MFMA kernel (0: 8 waves x 32 rows, 1: 4 x 64)
  */
-#define MSGL_TUNE_DECODE_CHUNK 0
-#define MSGL_TUNE_SMALLQ_CHUNK 1
+#define MSGL_TUNE_SEGMENTS 0
+#define MSGL_TUNE_MIN_SEGMENT 1
 #define MSGL_TUNE_SMALLQ_MAXCOLS 2
 #define MSGL_TUNE_PREFILL_VARIANT 3
 MSGL_API int msgl_set_tuning(int32_t knob, int64_t value);

@@ -28,15 +28,15 @@ int check_common(const void* q, const void* k_cache, const void* v_cache, const 
   return MSGL_OK;
 }
 
-int32_t decode_chunk(int64_t total_kv, int64_t n_kv, int64_t group) {
-  const int64_t t = g_tune[MSGL_TUNE_DECODE_CHUNK].load();
-  if (t >= 32) return (int32_t)(t / 32 * 32);
-  return msgl::splitkv_default_chunk(total_kv, n_kv, group);
+int32_t min_segment() {
+  const int64_t t = g_tune[MSGL_TUNE_MIN_SEGMENT].load();
+  if (t >= 64) return (int32_t)(t / 64 * 64);
+  return msgl::kSplitKvMinSegment;
 }
-int32_t smallq_chunk(int64_t total_kv, int64_t n_kv, int64_t cols) {
-  const int64_t t = g_tune[MSGL_TUNE_SMALLQ_CHUNK].load();
-  if (t >= 32) return (int32_t)(t / 32 * 32);
-  return msgl::splitkv_default_chunk(total_kv, n_kv, cols);
+int32_t segments(int64_t total_kv, int64_t n_kv, int64_t head_dim, int64_t cols) {
+  const int64_t t = g_tune[MSGL_TUNE_SEGMENTS].load();
+  if (t >= 1) return (int32_t)(t < (1 << 20) ? t : (1 << 20));
+  return msgl::splitkv_default_segments(total_kv, n_kv, head_dim, cols, min_segment());
 }
 int64_t smallq_max_cols() {
   const int64_t t = g_tune[MSGL_TUNE_SMALLQ_MAXCOLS].load();
@@ -104,8 +104,8 @@ size_t msgl_paged_decode_workspace_bytes(int64_t batch, int64_t total_kv, int64_
       num_q_heads % num_kv_heads != 0)
     return 0;
   const int64_t group = num_q_heads / num_kv_heads;
-  return msgl::splitkv_workspace_bytes(batch, total_kv, num_q_heads, num_kv_heads, head_dim, 1,
-                                       decode_chunk(total_kv, num_kv_heads, group));
+  return msgl::splitkv_workspace_bytes(batch, num_q_heads, num_kv_heads, head_dim, 1,
+                                       segments(total_kv, num_kv_heads, head_dim, group));
 }
 
 int msgl_paged_decode_attention(const void* q, const void* k_cache, const void* v_cache,
@@ -125,9 +125,9 @@ int msgl_paged_decode_attention(const void* q, const void* k_cache, const void* 
   if (group > 16) return MSGL_ERR_GROUP_TOO_LARGE;  // paged_decode_attention.cpp:54-57
   if (!kv_indptr || !num_kv_splits || (total_kv > 0 && !kv_indices)) return MSGL_ERR_NULL_POINTER;
   (void)max_kv_splits;  // split hints do not steer the cut (result is split-invariant)
-  const int32_t chunk = decode_chunk(total_kv, num_kv_heads, group);
-  const size_t need = msgl::splitkv_workspace_bytes(batch, total_kv, num_q_heads, num_kv_heads,
-                                                    head_dim, 1, chunk);
+  const int32_t n_seg = segments(total_kv, num_kv_heads, head_dim, group);
+  const size_t need =
+      msgl::splitkv_workspace_bytes(batch, num_q_heads, num_kv_heads, head_dim, 1, n_seg);
   if (!workspace || workspace_bytes < need || !aligned16(workspace)) return MSGL_ERR_WORKSPACE;
   msgl::SplitKvArgs a{};
   a.q = q;
@@ -150,7 +150,8 @@ int msgl_paged_decode_attention(const void* q, const void* k_cache, const void* 
   a.max_len_extend = 1;
   a.is_cross = 0;
   a.window = 0;
-  a.chunk = chunk;
+  a.n_seg = n_seg;
+  a.min_seg = min_segment();
   return msgl::launch_splitkv(a, static_cast<hipStream_t>(stream));
 }
 
@@ -168,8 +169,8 @@ size_t msgl_paged_prefill_workspace_bytes(int64_t batch, int64_t total_q, int64_
   const int64_t group = num_q_heads / num_kv_heads;
   if (!use_splitkv_route(group, max_len_extend)) return 0;
   return msgl::splitkv_workspace_bytes(
-      batch, total_kv, num_q_heads, num_kv_heads, head_dim, max_len_extend,
-      smallq_chunk(total_kv, num_kv_heads, group * max_len_extend));
+      batch, num_q_heads, num_kv_heads, head_dim, max_len_extend,
+      segments(total_kv, num_kv_heads, head_dim, group * max_len_extend));
 }
 
 int msgl_paged_prefill_attention(const void* q, const void* k_cache, const void* v_cache,
@@ -196,9 +197,9 @@ int msgl_paged_prefill_attention(const void* q, const void* k_cache, const void*
   const int64_t group = num_q_heads / num_kv_heads;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (use_splitkv_route(group, max_len_extend)) {
-    const int32_t chunk = smallq_chunk(total_kv, num_kv_heads, group * max_len_extend);
-    const size_t need = msgl::splitkv_workspace_bytes(batch, total_kv, num_q_heads, num_kv_heads,
-                                                      head_dim, max_len_extend, chunk);
+    const int32_t n_seg = segments(total_kv, num_kv_heads, head_dim, group * max_len_extend);
+    const size_t need = msgl::splitkv_workspace_bytes(batch, num_q_heads, num_kv_heads, head_dim,
+                                                      max_len_extend, n_seg);
     if (!workspace || workspace_bytes < need || !aligned16(workspace)) return MSGL_ERR_WORKSPACE;
     msgl::SplitKvArgs a{};
     a.q = q;
@@ -221,7 +222,8 @@ int msgl_paged_prefill_attention(const void* q, const void* k_cache, const void*
     a.max_len_extend = max_len_extend;
     a.is_cross = is_cross_attention ? 1 : 0;
     a.window = sliding_window_size;
-    a.chunk = chunk;
+    a.n_seg = n_seg;
+    a.min_seg = min_segment();
     return msgl::launch_splitkv(a, s);
   }
   msgl::PrefillArgs a{};

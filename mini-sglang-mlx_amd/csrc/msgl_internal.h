@@ -32,13 +32,17 @@ struct SplitKvArgs {
   float sm_scale;
   int32_t max_len_extend;  // 1 for decode
   int32_t is_cross, window;
-  int32_t chunk;  // tokens per work item, multiple of 32
+  int32_t n_seg;    // segments the visible token stream is cut into
+  int32_t min_seg;  // smallest segment length in tokens, multiple of 64
 };
 // largest q_len * group the split-K kernel is instantiated for
 constexpr int kSplitKvMaxCols = 64;
-int splitkv_default_chunk(int64_t total_kv, int64_t n_kv, int64_t cols);
-size_t splitkv_workspace_bytes(int64_t batch, int64_t total_kv, int64_t n_q, int64_t n_kv,
-                               int64_t head_dim, int64_t max_len_extend, int32_t chunk);
+constexpr int kSplitKvMinSegment = 128;
+// one resident round of workgroups for this shape, capped so segments keep min_seg tokens
+int splitkv_default_segments(int64_t total_kv, int64_t n_kv, int64_t head_dim, int64_t cols,
+                             int32_t min_seg);
+size_t splitkv_workspace_bytes(int64_t batch, int64_t n_q, int64_t n_kv, int64_t head_dim,
+                               int64_t max_len_extend, int32_t n_seg);
 int launch_splitkv(const SplitKvArgs& a, hipStream_t stream);
 
 // ---- paged_prefill.hip -------------------------------------------------------------

@@ -6,11 +6,22 @@
 // (mini-sglang-mlx-kernel/csrc/paged_decode_attention.metal:313-586) and, for short
 // extends, paged_prefill_attention (paged_prefill_attention.metal:382-640).
 //
-// Shape of the computation
-//   work item  = (request, kv head, chunk of `chunk` consecutive visible tokens), one wave64.
-//   columns    = the q rows that share this kv head: col = q_idx * group + head_in_group,
+// Work decomposition
+//   The visible keys of all requests, in CSR order, form one token stream.  It is cut
+//   into `n_seg` equal segments (the count is chosen on the host so that all workgroups
+//   are resident at once: one round, no tail).  A workgroup owns one segment and NW
+//   adjacent kv heads, one wave64 per head; its waves walk the same tokens, so the
+//   workgroup touches NW*256-byte stretches of every slot row together.  A segment may
+//   cross request boundaries: the wave finishes one request's share (writing bf16 output
+//   directly if it covered the whole request, otherwise a normalised fp32 partial + base-2
+//   LSE) and continues with the next.  splitkv_merge_kernel combines the partials.
+//   The host never reads device metadata: every wave derives its segment from kv_indptr
+//   (and qo_indptr / prefix_lens) with a wave-wide prefix sum.
+//
+// Inner product shapes (one wave, one kv head)
+//   columns    = the q rows sharing this kv head: col = q_idx * group + head_in_group,
 //                padded to NCT tiles of 16 (the MFMA N dimension).  Every K / V row is
-//                therefore read once per kv head, whatever the group size or q_len.
+//                read once per kv head, whatever the group size or q_len.
 //   S^T        = K_tile (16 tokens x D) * Q^T        -> mfma 16x16x32, tokens on M
 //   O^T       += V_tile^T (D x 32 tokens) * P^T      -> mfma 16x16x32, tokens on K
 //   Both products keep "column" on l%16 of the accumulator, so the softmax state, the
@@ -20,14 +31,11 @@
 //   turned into the token-contiguous MFMA operand by an in-lane 8x8 transpose of 16-bit
 //   values (v_perm_b32); the token order inside an MFMA is chosen so that it matches the
 //   accumulator layout of S^T, which is legal because the contraction is a sum.
-//   Item -> (request, chunk) is recomputed by every wave from kv_indptr with a wave-wide
-//   prefix sum: the host never reads device metadata, so the grid is the host-known upper
-//   bound ceil(total_kv / chunk) + batch and surplus waves exit.
-//   Requests that fit one chunk write bf16 output directly; others write a normalised fp32
-//   partial + base-2 LSE, merged by splitkv_merge_kernel.
 //
 // Algorithmic HBM bytes per visible token and kv head: 2 * D * 2 (one K row + one V row)
 // plus 4 bytes of kv_indices per token.
+#include <atomic>
+
 #include "msgl_device.h"
 #include "msgl_internal.h"
 
@@ -43,12 +51,14 @@ struct SplitKvParams {
   const int32_t* qo_indptr;
   const int32_t* prefix_lens;
   uint16_t* out;
-  float* part_o;           // [max_items][n_kv][cols_pad][D]
-  float* part_lse;         // [max_items][n_kv][cols_pad]
-  int32_t* req_item_base;  // [batch] first item of a request (written by its chunk 0)
+  float* part_o;        // [n_seg + batch][n_kv][cols][D]
+  float* part_lse;      // [n_seg + batch][n_kv][cols]
+  int32_t* req_vstart;  // [batch] stream position of a request's first visible key
+  int32_t* seg_info;    // [0] = segment length the attention kernel used
   int64_t k_stride0, v_stride0;
   int32_t batch, n_q, n_kv, group;
-  int32_t max_items, cols_pad, max_len_extend, chunk;
+  int32_t head_groups;  // n_kv / waves per workgroup
+  int32_t n_seg, min_seg, cols, max_len_extend;
   int32_t is_cross, window;
   float scale_log2e;
 };
@@ -86,33 +96,54 @@ __device__ __forceinline__ ReqInfo request_info(const SplitKvParams& p, int b) {
   return r;
 }
 
-__device__ __forceinline__ int32_t num_chunks(const ReqInfo& r, int chunk) {
-  return (r.hi - r.lo + chunk - 1) / chunk;
+__device__ __forceinline__ int segment_length(int total, int n_seg, int min_seg) {
+  const int even = ((total + n_seg - 1) / n_seg + 63) / 64 * 64;
+  return max(even, min_seg);
 }
 
-// Wave-cooperative search: which request owns work item `item`?  Returns false when the
-// item lies beyond the last request.  All lanes must call.
-__device__ __forceinline__ bool locate_item(const SplitKvParams& p, int item, int* req,
-                                            int* chunk_idx, int* item_base) {
+// Wave-cooperative: length of the visible token stream, and the request that holds stream
+// position `seg * seg_len` together with the stream position of that request's first key.
+// Returns false when the segment starts beyond the stream.  All lanes must call.
+__device__ __forceinline__ bool locate_segment(const SplitKvParams& p, int seg, int* seg_len,
+                                               int* total_out, int* req, int* req_vstart) {
   const int lane = lane_id();
-  int base = 0;
+  int total = 0, n = 0, incl = 0;
   for (int b0 = 0; b0 < p.batch; b0 += kWave) {
     const int b = b0 + lane;
-    int n = 0;
-    if (b < p.batch) n = num_chunks(request_info(p, b), p.chunk);
-    const int incl = wave_inclusive_scan(n);
-    const int total = __shfl(incl, kWave - 1, kWave);
-    if (item < base + total) {
+    n = 0;
+    if (b < p.batch) {
+      const ReqInfo r = request_info(p, b);
+      n = r.hi - r.lo;
+    }
+    incl = wave_inclusive_scan(n);
+    total += __shfl(incl, kWave - 1, kWave);
+  }
+  const int len = segment_length(total, p.n_seg, p.min_seg);
+  *seg_len = len;
+  *total_out = total;
+  const int pos = seg * len;
+  if (pos >= total) return false;
+  int base = 0;
+  for (int b0 = 0; b0 < p.batch; b0 += kWave) {
+    if (p.batch > kWave) {  // more than one batch of requests: recompute this batch
+      const int b = b0 + lane;
+      n = 0;
+      if (b < p.batch) {
+        const ReqInfo r = request_info(p, b);
+        n = r.hi - r.lo;
+      }
+      incl = wave_inclusive_scan(n);
+    }
+    const int batch_total = __shfl(incl, kWave - 1, kWave);
+    if (pos < base + batch_total) {
       const int first = base + incl - n;
-      const bool hit = (item >= first) && (item < first + n);
-      const unsigned long long m = __ballot(hit);
-      const int src = __ffsll((long long)m) - 1;
+      const bool hit = (pos >= first) && (pos < first + n);
+      const int src = __ffsll((long long)__ballot(hit)) - 1;
       *req = b0 + src;
-      *item_base = __shfl(first, src, kWave);
-      *chunk_idx = item - *item_base;
+      *req_vstart = __shfl(first, src, kWave);
       return true;
     }
-    base += total;
+    base += batch_total;
   }
   return false;
 }
@@ -123,256 +154,276 @@ struct KvTile {
   u32x4_t v[D / 128][8];  // [128-wide half of D][token j of the lane group]: raw V segments
 };
 
+// Two waves per SIMD where the register budget allows it (256 VGPRs each).
 template <int D, int NCT>
-__global__ __launch_bounds__(64) void splitkv_attention_kernel(SplitKvParams p) {
+constexpr int splitkv_min_waves() { return (D == 128 && NCT == 1) ? 2 : 1; }
+
+template <int D, int NCT, int NW>
+__global__ __launch_bounds__(64 * NW, (splitkv_min_waves<D, NCT>())) void splitkv_attention_kernel(SplitKvParams p) {
   constexpr int KS = D / 32;   // k-steps of the QK product
   constexpr int VH = D / 128;  // 128-wide halves of D in the PV product
   const int lane = lane_id();
   const int t16 = lane & 15;
   const int g = lane >> 4;
 
-  const int item = blockIdx.x / p.n_kv;
-  const int kvh = blockIdx.x - item * p.n_kv;
-  int b, chunk_idx, item_base;
-  if (!locate_item(p, item, &b, &chunk_idx, &item_base)) return;
-  const ReqInfo r = request_info(p, b);
-  const int n_items = num_chunks(r, p.chunk);
-  if (chunk_idx == 0 && kvh == 0 && lane == 0) p.req_item_base[b] = item_base;
+  const int seg = blockIdx.x / p.head_groups;
+  const int kvh = (blockIdx.x - seg * p.head_groups) * NW + (threadIdx.x >> 6);
+  int seg_len, total, cur_b, vs;
+  if (!locate_segment(p, seg, &seg_len, &total, &cur_b, &vs)) return;
+  if (blockIdx.x == 0 && threadIdx.x == 0) p.seg_info[0] = seg_len;
+  cur_b = __builtin_amdgcn_readfirstlane(cur_b);
+  vs = __builtin_amdgcn_readfirstlane(vs);
+  int vpos = seg * seg_len;
+  const int seg_end = min(vpos + seg_len, total);
 
-  const int t_begin = r.lo + chunk_idx * p.chunk;
-  const int t_end = min(r.hi, t_begin + p.chunk);
-  const int ncols = r.q_len * p.group;
-
-  // ---- Q operand and per-column visibility bounds --------------------------------
-  bf16x8_t qreg[NCT][KS];
-  int col_lo[NCT], col_hi[NCT];
-  int all_lo = 0, all_hi = 0x7fffffff;  // tile is mask-free iff inside [all_lo, all_hi]
-#pragma unroll
-  for (int ct = 0; ct < NCT; ++ct) {
-    const int col = ct * 16 + t16;
-    const bool valid = col < ncols;
-    const int qi = valid ? col / p.group : 0;
-    const int hh = valid ? col - qi * p.group : 0;
-    const uint16_t* qrow =
-        p.q + ((int64_t)(r.q_start + qi) * p.n_q + kvh * p.group + hh) * D + g * 8;
-#pragma unroll
-    for (int c = 0; c < KS; ++c) {
-      u32x4_t raw = {0u, 0u, 0u, 0u};
-      if (valid) raw = ld_global_b128(qrow + c * 32);
-      qreg[ct][c] = as_bf16x8(raw);
-    }
-    const int qpos = r.prefix + qi;
-    int lo = (p.window > 0) ? qpos - p.window + 1 : 0;
-    int hi = p.is_cross ? r.kv_len - 1 : min(qpos, r.kv_len - 1);
-    hi = min(hi, t_end - 1);
-    if (valid) {
-      all_lo = max(all_lo, lo);
-      all_hi = min(all_hi, hi);
-    } else {
-      lo = 1;
-      hi = 0;
-    }
-    col_lo[ct] = lo;
-    col_hi[ct] = hi;
-  }
-#pragma unroll
-  for (int off = 1; off < 16; off <<= 1) {
-    all_lo = max(all_lo, __shfl_xor(all_lo, off, kWave));
-    all_hi = min(all_hi, __shfl_xor(all_hi, off, kWave));
-  }
-  all_lo = __builtin_amdgcn_readfirstlane(all_lo);
-  all_hi = __builtin_amdgcn_readfirstlane(all_hi);
-
-  // ---- accumulators ------------------------------------------------------------------
-  f32x4_t oacc[NCT][VH][8];
-  float m_run[NCT], l_run[NCT];
-#pragma unroll
-  for (int ct = 0; ct < NCT; ++ct) {
-    m_run[ct] = kNegInf;
-    l_run[ct] = 0.f;
-#pragma unroll
-    for (int hf = 0; hf < VH; ++hf)
-#pragma unroll
-      for (int n = 0; n < 8; ++n) oacc[ct][hf][n] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-  }
-
-  const int32_t* idx_base = p.kv_indices + r.kv_start;
   const uint16_t* kbase = p.k_cache + (int64_t)kvh * D + g * 8;
   const uint16_t* vbase = p.v_cache + (int64_t)kvh * D + t16 * 8;
-  const int last_tok = t_end - 1;
 
-  // slot ids of the two K rows this lane loads in a 32-token tile starting at tb
-  auto load_idx = [&](int tb, int& s0, int& s1) {
-    s0 = idx_base[min(tb + t16, last_tok)];
-    s1 = idx_base[min(tb + 16 + t16, last_tok)];
-  };
-  auto load_tile = [&](KvTile<D>& t, int s0, int s1) {
-#pragma unroll
-    for (int c = 0; c < KS; ++c) {
-      t.k[0][c] = ld_global_b128(kbase + (int64_t)s0 * p.k_stride0 + c * 32);
-      t.k[1][c] = ld_global_b128(kbase + (int64_t)s1 * p.k_stride0 + c * 32);
+  while (vpos < seg_end) {
+    const ReqInfo r = request_info(p, cur_b);
+    const int vlen = r.hi - r.lo;
+    if (vlen == 0) {
+      ++cur_b;
+      continue;
     }
-    // V rows of this lane group: tokens 4g+j (j<4) of sub-tile 0, then of sub-tile 1;
-    // their slot ids sit in lanes 4g+j of the K index registers.
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int src = 4 * g + (j & 3);
-      const int slot = __shfl(j < 4 ? s0 : s1, src, kWave);
-      const uint16_t* vrow = vbase + (int64_t)slot * p.v_stride0;
-#pragma unroll
-      for (int hf = 0; hf < VH; ++hf) t.v[hf][j] = ld_global_b128(vrow + hf * 128);
-    }
-  };
+    const int t_begin = r.lo + (vpos - vs);
+    const int t_end = min(r.hi, t_begin + (seg_end - vpos));
+    const bool whole = (t_begin == r.lo) && (t_end == r.hi);
+    if (t_begin == r.lo && kvh == 0 && lane == 0) p.req_vstart[cur_b] = vs;
+    const int ncols = r.q_len * p.group;
 
-  auto compute_tile = [&](const KvTile<D>& t, int tb) {
-    // S^T[token][col] for the two 16-token sub-tiles
-    f32x4_t s[2][NCT];
-#pragma unroll
-    for (int sub = 0; sub < 2; ++sub)
-#pragma unroll
-      for (int ct = 0; ct < NCT; ++ct) {
-        f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int c = 0; c < KS; ++c)
-          acc = mfma_16x16x32(as_bf16x8(t.k[sub][c]), qreg[ct][c], acc);
-        s[sub][ct] = acc;
-      }
-    const bool need_mask = (tb < all_lo) || (tb + 31 > all_hi);
-    uint32_t pb[NCT][4];
+    // ---- Q operand and per-column visibility bounds --------------------------------
+    bf16x8_t qreg[NCT][KS];
+    int col_lo[NCT], col_hi[NCT];
+    int all_lo = 0, all_hi = 0x7fffffff;  // tile is mask-free iff inside [all_lo, all_hi]
 #pragma unroll
     for (int ct = 0; ct < NCT; ++ct) {
-      float x[2][4];
+      const int col = ct * 16 + t16;
+      const bool valid = col < ncols;
+      const int qi = valid ? col / p.group : 0;
+      const int hh = valid ? col - qi * p.group : 0;
+      const uint16_t* qrow =
+          p.q + ((int64_t)(r.q_start + qi) * p.n_q + kvh * p.group + hh) * D + g * 8;
+#pragma unroll
+      for (int c = 0; c < KS; ++c) {
+        u32x4_t raw = {0u, 0u, 0u, 0u};
+        if (valid) raw = ld_global_b128(qrow + c * 32);
+        qreg[ct][c] = as_bf16x8(raw);
+      }
+      const int qpos = r.prefix + qi;
+      int lo = (p.window > 0) ? qpos - p.window + 1 : 0;
+      int hi = p.is_cross ? r.kv_len - 1 : min(qpos, r.kv_len - 1);
+      hi = min(hi, t_end - 1);
+      if (valid) {
+        all_lo = max(all_lo, lo);
+        all_hi = min(all_hi, hi);
+      } else {
+        lo = 1;
+        hi = 0;
+      }
+      col_lo[ct] = lo;
+      col_hi[ct] = hi;
+    }
+#pragma unroll
+    for (int off = 1; off < 16; off <<= 1) {
+      all_lo = max(all_lo, __shfl_xor(all_lo, off, kWave));
+      all_hi = min(all_hi, __shfl_xor(all_hi, off, kWave));
+    }
+    all_lo = __builtin_amdgcn_readfirstlane(all_lo);
+    all_hi = __builtin_amdgcn_readfirstlane(all_hi);
+
+    // ---- accumulators ----------------------------------------------------------------
+    f32x4_t oacc[NCT][VH][8];
+    float m_run[NCT], l_run[NCT];
+#pragma unroll
+    for (int ct = 0; ct < NCT; ++ct) {
+      m_run[ct] = kNegInf;
+      l_run[ct] = 0.f;
+#pragma unroll
+      for (int hf = 0; hf < VH; ++hf)
+#pragma unroll
+        for (int n = 0; n < 8; ++n) oacc[ct][hf][n] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    }
+
+    const int32_t* idx_base = p.kv_indices + r.kv_start;
+    const int last_tok = t_end - 1;
+
+    // slot ids of the two K rows this lane loads in a 32-token tile starting at tb
+    auto load_idx = [&](int tb, int& s0, int& s1) {
+      s0 = idx_base[min(tb + t16, last_tok)];
+      s1 = idx_base[min(tb + 16 + t16, last_tok)];
+    };
+    auto load_tile = [&](KvTile<D>& t, int s0, int s1) {
+#pragma unroll
+      for (int c = 0; c < KS; ++c) {
+        t.k[0][c] = ld_global_b128(kbase + (int64_t)s0 * p.k_stride0 + c * 32);
+        t.k[1][c] = ld_global_b128(kbase + (int64_t)s1 * p.k_stride0 + c * 32);
+      }
+      // V rows of this lane group: tokens 4g+j (j<4) of sub-tile 0, then of sub-tile 1;
+      // their slot ids sit in lanes 4g+j of the K index registers.
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int src = 4 * g + (j & 3);
+        const int slot = __shfl(j < 4 ? s0 : s1, src, kWave);
+        const uint16_t* vrow = vbase + (int64_t)slot * p.v_stride0;
+#pragma unroll
+        for (int hf = 0; hf < VH; ++hf) t.v[hf][j] = ld_global_b128(vrow + hf * 128);
+      }
+    };
+
+    auto compute_tile = [&](const KvTile<D>& t, int tb) {
+      // S^T[token][col] for the two 16-token sub-tiles
+      f32x4_t s[2][NCT];
 #pragma unroll
       for (int sub = 0; sub < 2; ++sub)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) x[sub][i] = s[sub][ct][i] * p.scale_log2e;
-      if (need_mask) {
+        for (int ct = 0; ct < NCT; ++ct) {
+          f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int c = 0; c < KS; ++c)
+            acc = mfma_16x16x32(as_bf16x8(t.k[sub][c]), qreg[ct][c], acc);
+          s[sub][ct] = acc;
+        }
+      const bool need_mask = (tb < all_lo) || (tb + 31 > all_hi);
+      uint32_t pb[NCT][4];
+#pragma unroll
+      for (int ct = 0; ct < NCT; ++ct) {
+        float x[2][4];
+#pragma unroll
+        for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) x[sub][i] = s[sub][ct][i] * p.scale_log2e;
+        if (need_mask) {
+#pragma unroll
+          for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const int tok = tb + sub * 16 + 4 * g + i;
+              if (tok < col_lo[ct] || tok > col_hi[ct]) x[sub][i] = kNegInf;
+            }
+        }
+        float mx = fmaxf(fmaxf(fmaxf(x[0][0], x[0][1]), fmaxf(x[0][2], x[0][3])),
+                         fmaxf(fmaxf(x[1][0], x[1][1]), fmaxf(x[1][2], x[1][3])));
+        mx = wave_max_xor(mx, 16);
+        mx = wave_max_xor(mx, 32);
+        const float m_new = fmaxf(m_run[ct], mx);
+        const float m_safe = (m_new == kNegInf) ? 0.f : m_new;
+        const float alpha = fast_exp2(m_run[ct] - m_safe);
+        m_run[ct] = m_new;
+        float psum = 0.f;
 #pragma unroll
         for (int sub = 0; sub < 2; ++sub)
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            const int tok = tb + sub * 16 + 4 * g + i;
-            if (tok < col_lo[ct] || tok > col_hi[ct]) x[sub][i] = kNegInf;
+            x[sub][i] = fast_exp2(x[sub][i] - m_safe);
+            psum += x[sub][i];
           }
-      }
-      float mx = fmaxf(fmaxf(fmaxf(x[0][0], x[0][1]), fmaxf(x[0][2], x[0][3])),
-                       fmaxf(fmaxf(x[1][0], x[1][1]), fmaxf(x[1][2], x[1][3])));
-      mx = wave_max_xor(mx, 16);
-      mx = wave_max_xor(mx, 32);
-      const float m_new = fmaxf(m_run[ct], mx);
-      const float m_safe = (m_new == kNegInf) ? 0.f : m_new;
-      const float alpha = fast_exp2(m_run[ct] - m_safe);
-      m_run[ct] = m_new;
-      float psum = 0.f;
+        l_run[ct] = l_run[ct] * alpha + psum;
+        pb[ct][0] = pack_bf16x2(x[0][0], x[0][1]);
+        pb[ct][1] = pack_bf16x2(x[0][2], x[0][3]);
+        pb[ct][2] = pack_bf16x2(x[1][0], x[1][1]);
+        pb[ct][3] = pack_bf16x2(x[1][2], x[1][3]);
+        if (__any(alpha != 1.0f)) {
 #pragma unroll
-      for (int sub = 0; sub < 2; ++sub)
+          for (int hf = 0; hf < VH; ++hf)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          x[sub][i] = fast_exp2(x[sub][i] - m_safe);
-          psum += x[sub][i];
-        }
-      l_run[ct] = l_run[ct] * alpha + psum;
-      pb[ct][0] = pack_bf16x2(x[0][0], x[0][1]);
-      pb[ct][1] = pack_bf16x2(x[0][2], x[0][3]);
-      pb[ct][2] = pack_bf16x2(x[1][0], x[1][1]);
-      pb[ct][3] = pack_bf16x2(x[1][2], x[1][3]);
-      if (__any(alpha != 1.0f)) {
-#pragma unroll
-        for (int hf = 0; hf < VH; ++hf)
-#pragma unroll
-          for (int n = 0; n < 8; ++n) oacc[ct][hf][n] *= alpha;
-      }
-    }
-    // O^T += V^T P^T.  MFMA n of half hf produces d = hf*128 + 8*row + n on row = l%16.
-#pragma unroll
-    for (int hf = 0; hf < VH; ++hf)
-#pragma unroll
-      for (int n = 0; n < 8; ++n) {
-        u32x4_t vt;
-#pragma unroll
-        for (int qd = 0; qd < 4; ++qd) {
-          const uint32_t a = t.v[hf][2 * qd][n >> 1];
-          const uint32_t c = t.v[hf][2 * qd + 1][n >> 1];
-          vt[qd] = (n & 1) ? pack_hi16(a, c) : pack_lo16(a, c);
-        }
-#pragma unroll
-        for (int ct = 0; ct < NCT; ++ct) {
-          const u32x4_t pv = {pb[ct][0], pb[ct][1], pb[ct][2], pb[ct][3]};
-          oacc[ct][hf][n] = mfma_16x16x32(as_bf16x8(vt), as_bf16x8(pv), oacc[ct][hf][n]);
+            for (int n = 0; n < 8; ++n) oacc[ct][hf][n] *= alpha;
         }
       }
-  };
+      // O^T += V^T P^T.  MFMA n of half hf produces d = hf*128 + 8*row + n on row = l%16.
+#pragma unroll
+      for (int hf = 0; hf < VH; ++hf)
+#pragma unroll
+        for (int n = 0; n < 8; ++n) {
+          u32x4_t vt;
+#pragma unroll
+          for (int qd = 0; qd < 4; ++qd) {
+            const uint32_t a = t.v[hf][2 * qd][n >> 1];
+            const uint32_t c = t.v[hf][2 * qd + 1][n >> 1];
+            vt[qd] = (n & 1) ? pack_hi16(a, c) : pack_lo16(a, c);
+          }
+#pragma unroll
+          for (int ct = 0; ct < NCT; ++ct) {
+            const u32x4_t pv = {pb[ct][0], pb[ct][1], pb[ct][2], pb[ct][3]};
+            oacc[ct][hf][n] = mfma_16x16x32(as_bf16x8(vt), as_bf16x8(pv), oacc[ct][hf][n]);
+          }
+        }
+    };
 
-  // ---- main loop: two register tiles; slot ids are fetched two tiles ahead so that
-  // issuing the next tile's loads never waits on the tile still in flight ----------------
-  const int n_tiles = (t_end - t_begin + 31) / 32;
-  KvTile<D> ta, tb_;
-  int i0a, i0b, i1a, i1b;
-  load_idx(t_begin, i0a, i0b);
-  load_idx(t_begin + 32, i1a, i1b);
-  load_tile(ta, i0a, i0b);
-  load_idx(t_begin + 64, i0a, i0b);
-  for (int t = 0; t < n_tiles; t += 2) {
-    const int tok = t_begin + t * 32;
-    if (t + 1 < n_tiles) load_tile(tb_, i1a, i1b);
-    load_idx(tok + 96, i1a, i1b);
-    compute_tile(ta, tok);
-    if (t + 1 < n_tiles) {
-      if (t + 2 < n_tiles) load_tile(ta, i0a, i0b);
+    // ---- tile loop: two register tiles, slot ids fetched two tiles ahead.  Every load in
+    // the loop body is unconditional (tokens past the range clamp to its last token and
+    // are masked), so the number of loads in flight at each wait is a compile-time
+    // constant and the next tile stays in flight while the current one is computed. ----
+    const int n_pairs = (t_end - t_begin + 63) / 64;
+    KvTile<D> ta, tb_;
+    int i0a, i0b, i1a, i1b;
+    load_idx(t_begin, i0a, i0b);
+    load_idx(t_begin + 32, i1a, i1b);
+    load_tile(ta, i0a, i0b);
+    load_idx(t_begin + 64, i0a, i0b);
+    for (int pr = 0; pr < n_pairs; ++pr) {
+      const int tok = t_begin + pr * 64;
+      load_tile(tb_, i1a, i1b);
+      load_idx(tok + 96, i1a, i1b);
+      compute_tile(ta, tok);
+      load_tile(ta, i0a, i0b);
       load_idx(tok + 128, i0a, i0b);
       compute_tile(tb_, tok + 32);
     }
-  }
 
-  // ---- epilogue ----------------------------------------------------------------------
-  const bool direct = (n_items == 1);
+    // ---- this request's share is done: write output or partial -------------------------
 #pragma unroll
-  for (int ct = 0; ct < NCT; ++ct) {
-    float l = l_run[ct];
-    l += __shfl_xor(l, 16, kWave);
-    l += __shfl_xor(l, 32, kWave);
-    const float inv = (l > 0.f) ? 1.0f / l : 0.f;
-    const int col = ct * 16 + t16;
-    if (col >= ncols) continue;
-    const int qi = col / p.group;
-    const int hh = col - qi * p.group;
-    if (direct) {
-      uint16_t* orow = p.out + ((int64_t)(r.q_start + qi) * p.n_q + kvh * p.group + hh) * D;
+    for (int ct = 0; ct < NCT; ++ct) {
+      float l = l_run[ct];
+      l += __shfl_xor(l, 16, kWave);
+      l += __shfl_xor(l, 32, kWave);
+      const float inv = (l > 0.f) ? 1.0f / l : 0.f;
+      const int col = ct * 16 + t16;
+      if (col >= ncols) continue;
+      const int qi = col / p.group;
+      const int hh = col - qi * p.group;
+      if (whole) {
+        uint16_t* orow = p.out + ((int64_t)(r.q_start + qi) * p.n_q + kvh * p.group + hh) * D;
 #pragma unroll
-      for (int hf = 0; hf < VH; ++hf)
+        for (int hf = 0; hf < VH; ++hf)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          u32x4_t w;
+          for (int i = 0; i < 4; ++i) {
+            u32x4_t w;
 #pragma unroll
-          for (int n = 0; n < 4; ++n)
-            w[n] = pack_bf16x2(oacc[ct][hf][2 * n][i] * inv, oacc[ct][hf][2 * n + 1][i] * inv);
-          st_global_b128(orow + hf * 128 + (4 * g + i) * 8, w);
-        }
-    } else {
-      const int64_t prow = ((int64_t)item * p.n_kv + kvh) * p.cols_pad + col;
-      float* po = p.part_o + prow * D;
-#pragma unroll
-      for (int hf = 0; hf < VH; ++hf)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          f32x4_t w0, w1;
-#pragma unroll
-          for (int n = 0; n < 4; ++n) {
-            w0[n] = oacc[ct][hf][n][i] * inv;
-            w1[n] = oacc[ct][hf][4 + n][i] * inv;
+            for (int n = 0; n < 4; ++n)
+              w[n] = pack_bf16x2(oacc[ct][hf][2 * n][i] * inv, oacc[ct][hf][2 * n + 1][i] * inv);
+            st_global_b128(orow + hf * 128 + (4 * g + i) * 8, w);
           }
-          float* dst = po + hf * 128 + (4 * g + i) * 8;
-          *reinterpret_cast<f32x4_t*>(dst) = w0;
-          *reinterpret_cast<f32x4_t*>(dst + 4) = w1;
-        }
-      if (g == 0) p.part_lse[prow] = (l > 0.f) ? m_run[ct] + __log2f(l) : kNegInf;
+      } else {
+        const int64_t prow = ((int64_t)(seg + cur_b) * p.n_kv + kvh) * p.cols + col;
+        float* po = p.part_o + prow * D;
+#pragma unroll
+        for (int hf = 0; hf < VH; ++hf)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            f32x4_t w0, w1;
+#pragma unroll
+            for (int n = 0; n < 4; ++n) {
+              w0[n] = oacc[ct][hf][n][i] * inv;
+              w1[n] = oacc[ct][hf][4 + n][i] * inv;
+            }
+            float* dst = po + hf * 128 + (4 * g + i) * 8;
+            *reinterpret_cast<f32x4_t*>(dst) = w0;
+            *reinterpret_cast<f32x4_t*>(dst + 4) = w1;
+          }
+        if (g == 0) p.part_lse[prow] = (l > 0.f) ? m_run[ct] + __log2f(l) : kNegInf;
+      }
     }
+
+    vpos += t_end - t_begin;
+    vs += vlen;
+    ++cur_b;
   }
 }
 
-// One wave per (request, query, q head): merge the request's partials by base-2 LSE.
-// Requests without visible keys (or empty) get zeros; single-item requests were written
-// by the attention kernel itself.
+// One wave per (request, query, q head): merge the partials of the segments that share
+// the request, by base-2 LSE.  Requests without visible keys get zeros; requests that sat
+// inside one segment were written by the attention kernel itself.
 template <int D>
 __global__ __launch_bounds__(64) void splitkv_merge_kernel(SplitKvParams p) {
   const int b = blockIdx.x / p.max_len_extend;
@@ -381,20 +432,23 @@ __global__ __launch_bounds__(64) void splitkv_merge_kernel(SplitKvParams p) {
   const int lane = lane_id();
   const ReqInfo r = request_info(p, b);
   if (qi >= r.q_len) return;
-  const int n_items = num_chunks(r, p.chunk);
-  if (n_items == 1) return;
   constexpr int PER = D / kWave;  // consecutive floats per lane
   uint16_t* orow = p.out + ((int64_t)(r.q_start + qi) * p.n_q + hq) * D + lane * PER;
-  if (n_items == 0) {
+  const int vlen = r.hi - r.lo;
+  if (vlen == 0) {
 #pragma unroll
     for (int e = 0; e < PER; ++e) orow[e] = 0;
     return;
   }
+  const int seg_len = p.seg_info[0];
+  const int vs = p.req_vstart[b];
+  const int s_first = vs / seg_len;
+  const int n_items = (vs + vlen - 1) / seg_len - s_first + 1;
+  if (n_items == 1) return;
   const int kvh = hq / p.group;
   const int col = qi * p.group + (hq - kvh * p.group);
-  const int base = p.req_item_base[b];
-  const int64_t stride = (int64_t)p.n_kv * p.cols_pad;
-  const int64_t row0 = ((int64_t)base * p.n_kv + kvh) * p.cols_pad + col;
+  const int64_t stride = (int64_t)p.n_kv * p.cols;
+  const int64_t row0 = ((int64_t)(s_first + b) * p.n_kv + kvh) * p.cols + col;
 
   float mx = kNegInf;
   for (int it = lane; it < n_items; it += kWave) mx = fmaxf(mx, p.part_lse[row0 + it * stride]);
@@ -405,12 +459,32 @@ __global__ __launch_bounds__(64) void splitkv_merge_kernel(SplitKvParams p) {
   for (int e = 0; e < PER; ++e) acc[e] = 0.f;
   float wsum = 0.f;
   if (mx > kNegInf) {
-    for (int it = 0; it < n_items; ++it) {
-      const float w = fast_exp2(p.part_lse[row0 + it * stride] - mx);
-      const float* src = p.part_o + (row0 + it * stride) * D + lane * PER;
+    int it = 0;
+    for (; it + 4 <= n_items; it += 4) {  // four independent partial rows in flight
+      float w[4], v[4][PER];
 #pragma unroll
-      for (int e = 0; e < PER; ++e) acc[e] += w * src[e];
-      wsum += w;
+      for (int u = 0; u < 4; ++u) {
+        const int64_t row = row0 + (it + u) * stride;
+        w[u] = p.part_lse[row];
+        const float* src = p.part_o + row * D + lane * PER;
+#pragma unroll
+        for (int e = 0; e < PER; ++e) v[u][e] = src[e];
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const float wu = fast_exp2(w[u] - mx);
+#pragma unroll
+        for (int e = 0; e < PER; ++e) acc[e] += wu * v[u][e];
+        wsum += wu;
+      }
+    }
+    for (; it < n_items; ++it) {
+      const int64_t row = row0 + it * stride;
+      const float wu = fast_exp2(p.part_lse[row] - mx);
+      const float* src = p.part_o + row * D + lane * PER;
+#pragma unroll
+      for (int e = 0; e < PER; ++e) acc[e] += wu * src[e];
+      wsum += wu;
     }
   }
   const float inv = (wsum > 0.f) ? 1.0f / wsum : 0.f;
@@ -419,63 +493,111 @@ __global__ __launch_bounds__(64) void splitkv_merge_kernel(SplitKvParams p) {
     *reinterpret_cast<uint32_t*>(orow + e) = pack_bf16x2(acc[e] * inv, acc[e + 1] * inv);
 }
 
-int64_t max_items_for(int64_t batch, int64_t total_kv, int32_t chunk) {
-  return (total_kv + chunk - 1) / chunk + batch;
-}
-int cols_pad_for(int64_t cols) { return (int)((cols + 15) / 16 * 16); }
+int waves_per_group(int64_t n_kv) { return (n_kv % 4 == 0) ? 4 : (n_kv % 2 == 0) ? 2 : 1; }
 
-template <int D>
-int launch_d(const SplitKvParams& p, int nct, int64_t n_blocks, hipStream_t stream) {
-  const dim3 grid((unsigned)n_blocks), block(64);
+// Workgroups of a kernel variant that one GPU holds at the same time.
+template <typename K>
+int resident_blocks(K kernel, int block_threads, std::atomic<int>& cache) {
+  int v = cache.load();
+  if (v > 0) return v;
+  int dev = 0, cus = 0, per_cu = 0;
+  if (hipGetDevice(&dev) != hipSuccess ||
+      hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+      hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, block_threads, 0) != hipSuccess ||
+      cus <= 0 || per_cu <= 0) {
+    (void)hipGetLastError();
+    return 512;  // MI355X: 256 CUs x 2
+  }
+  v = cus * per_cu;
+  cache.store(v);
+  return v;
+}
+
+template <int D, int NCT, int NW>
+int resident_for() {
+  static std::atomic<int> cache{0};
+  return resident_blocks(splitkv_attention_kernel<D, NCT, NW>, 64 * NW, cache);
+}
+
+template <int D, int NW>
+int resident_dw(int nct) {
   switch (nct) {
-    case 1: hipLaunchKernelGGL((splitkv_attention_kernel<D, 1>), grid, block, 0, stream, p); break;
-    case 2: hipLaunchKernelGGL((splitkv_attention_kernel<D, 2>), grid, block, 0, stream, p); break;
-    case 3: hipLaunchKernelGGL((splitkv_attention_kernel<D, 3>), grid, block, 0, stream, p); break;
-    case 4: hipLaunchKernelGGL((splitkv_attention_kernel<D, 4>), grid, block, 0, stream, p); break;
+    case 1: return resident_for<D, 1, NW>();
+    case 2: return resident_for<D, 2, NW>();
+    case 3: return resident_for<D, 3, NW>();
+    default: return resident_for<D, 4, NW>();
+  }
+}
+
+int resident_any(int64_t head_dim, int nct, int nw) {
+  if (head_dim == 128) {
+    if (nw == 4) return resident_dw<128, 4>(nct);
+    if (nw == 2) return resident_dw<128, 2>(nct);
+    return resident_dw<128, 1>(nct);
+  }
+  if (nw == 4) return resident_dw<256, 4>(nct);
+  if (nw == 2) return resident_dw<256, 2>(nct);
+  return resident_dw<256, 1>(nct);
+}
+
+template <int D, int NW>
+int launch_dw(const SplitKvParams& p, int nct, hipStream_t stream) {
+  const dim3 grid((unsigned)(p.n_seg * p.head_groups)), block(64 * NW);
+  switch (nct) {
+    case 1: hipLaunchKernelGGL((splitkv_attention_kernel<D, 1, NW>), grid, block, 0, stream, p); break;
+    case 2: hipLaunchKernelGGL((splitkv_attention_kernel<D, 2, NW>), grid, block, 0, stream, p); break;
+    case 3: hipLaunchKernelGGL((splitkv_attention_kernel<D, 3, NW>), grid, block, 0, stream, p); break;
+    case 4: hipLaunchKernelGGL((splitkv_attention_kernel<D, 4, NW>), grid, block, 0, stream, p); break;
     default: return MSGL_ERR_SHAPE;
   }
   int rc = check_launch();
   if (rc != MSGL_OK) return rc;
   const dim3 mgrid((unsigned)(p.batch * p.max_len_extend), (unsigned)p.n_q);
-  hipLaunchKernelGGL((splitkv_merge_kernel<D>), mgrid, block, 0, stream, p);
+  hipLaunchKernelGGL((splitkv_merge_kernel<D>), mgrid, dim3(64), 0, stream, p);
   return check_launch();
 }
 
-}  // namespace
-
-int splitkv_default_chunk(int64_t total_kv, int64_t n_kv, int64_t cols) {
-  // Enough waves to fill 256 CUs several times over, while the fp32 partial a chunk
-  // writes (cols * D * 4 bytes per kv head) stays a few percent of the KV bytes it reads.
-  const int64_t target_waves = 8192;
-  int64_t chunk = (total_kv * n_kv + target_waves - 1) / target_waves;
-  const int64_t floor_for_partials = 32 * cols;  // partial bytes <= ~3 % of KV bytes
-  if (chunk < floor_for_partials) chunk = floor_for_partials;
-  if (chunk < 64) chunk = 64;
-  if (chunk > 4096) chunk = 4096;
-  return (int)((chunk + 31) / 32 * 32);
+template <int D>
+int launch_d(const SplitKvParams& p, int nct, int nw, hipStream_t stream) {
+  if (nw == 4) return launch_dw<D, 4>(p, nct, stream);
+  if (nw == 2) return launch_dw<D, 2>(p, nct, stream);
+  return launch_dw<D, 1>(p, nct, stream);
 }
 
-size_t splitkv_workspace_bytes(int64_t batch, int64_t total_kv, int64_t n_q, int64_t n_kv,
-                               int64_t head_dim, int64_t max_len_extend, int32_t chunk) {
-  const int64_t group = n_q / n_kv;
-  const int64_t items = max_items_for(batch, total_kv, chunk);
-  const int64_t rows = items * n_kv * cols_pad_for(group * max_len_extend);
+int nct_for(int64_t cols) { return (int)((cols + 15) / 16); }
+
+}  // namespace
+
+int splitkv_default_segments(int64_t total_kv, int64_t n_kv, int64_t head_dim, int64_t cols,
+                             int32_t min_seg) {
+  const int nw = waves_per_group(n_kv);
+  const int64_t head_groups = n_kv / nw;
+  const int resident = resident_any(head_dim, nct_for(cols), nw);
+  int64_t n_seg = resident / head_groups;  // one resident round
+  const int64_t by_len = (total_kv + min_seg - 1) / min_seg;
+  if (n_seg > by_len) n_seg = by_len;
+  if (n_seg < 1) n_seg = 1;
+  return (int)n_seg;
+}
+
+size_t splitkv_workspace_bytes(int64_t batch, int64_t n_q, int64_t n_kv, int64_t head_dim,
+                               int64_t max_len_extend, int32_t n_seg) {
+  const int64_t cols = n_q / n_kv * max_len_extend;
+  const int64_t rows = ((int64_t)n_seg + batch) * n_kv * cols;
   size_t bytes = (size_t)rows * (size_t)head_dim * sizeof(float);  // part_o
   bytes += (size_t)rows * sizeof(float);                           // part_lse
-  bytes += (size_t)batch * sizeof(int32_t);                        // req_item_base
+  bytes += (size_t)(batch + 4) * sizeof(int32_t);                  // req_vstart, seg_info
   return (bytes + 255) / 256 * 256 + 256;
 }
 
 int launch_splitkv(const SplitKvArgs& a, hipStream_t stream) {
   const int64_t group = a.n_q / a.n_kv;
   const int64_t cols = group * a.max_len_extend;
-  if (cols < 1 || cols > kSplitKvMaxCols || a.chunk < 32 || a.chunk % 32 != 0)
+  if (cols < 1 || cols > kSplitKvMaxCols || a.n_seg < 1 || a.min_seg < 64 || a.min_seg % 64 != 0)
     return MSGL_ERR_SHAPE;
-  const int64_t items = max_items_for(a.batch, a.total_kv, a.chunk);
-  const int64_t n_blocks = items * a.n_kv;
-  if (n_blocks > 0x7fffffffLL || a.batch * a.max_len_extend > 0x7fffffffLL)
-    return MSGL_ERR_SHAPE;
+  if (a.batch * a.max_len_extend > 0x7fffffffLL || a.total_kv > 0x7fffffffLL) return MSGL_ERR_SHAPE;
   if (a.batch == 0) return MSGL_OK;
+  const int nw = waves_per_group(a.n_kv);
 
   SplitKvParams p;
   p.q = static_cast<const uint16_t*>(a.q);
@@ -486,27 +608,30 @@ int launch_splitkv(const SplitKvArgs& a, hipStream_t stream) {
   p.qo_indptr = a.qo_indptr;
   p.prefix_lens = a.prefix_lens;
   p.out = static_cast<uint16_t*>(a.out);
-  p.cols_pad = cols_pad_for(cols);
-  const int64_t rows = items * a.n_kv * p.cols_pad;
+  p.cols = (int32_t)cols;
+  const int64_t rows = ((int64_t)a.n_seg + a.batch) * a.n_kv * cols;
   char* ws = static_cast<char*>(a.workspace);
   p.part_o = reinterpret_cast<float*>(ws);
   p.part_lse = reinterpret_cast<float*>(ws + (size_t)rows * a.head_dim * sizeof(float));
-  p.req_item_base = reinterpret_cast<int32_t*>(ws + (size_t)rows * (a.head_dim + 1) * sizeof(float));
+  p.req_vstart = reinterpret_cast<int32_t*>(ws + (size_t)rows * (a.head_dim + 1) * sizeof(float));
+  p.seg_info = p.req_vstart + a.batch;
   p.k_stride0 = a.k_stride0;
   p.v_stride0 = a.v_stride0;
   p.batch = (int32_t)a.batch;
   p.n_q = (int32_t)a.n_q;
   p.n_kv = (int32_t)a.n_kv;
   p.group = (int32_t)group;
-  p.max_items = (int32_t)items;
+  p.head_groups = (int32_t)(a.n_kv / nw);
+  p.n_seg = a.n_seg;
+  p.min_seg = a.min_seg;
   p.max_len_extend = a.max_len_extend;
-  p.chunk = a.chunk;
   p.is_cross = a.is_cross;
   p.window = a.window;
   p.scale_log2e = a.sm_scale * kLog2e;
-  const int nct = p.cols_pad / 16;
-  if (a.head_dim == 128) return launch_d<128>(p, nct, n_blocks, stream);
-  if (a.head_dim == 256) return launch_d<256>(p, nct, n_blocks, stream);
+  if ((int64_t)p.n_seg * p.head_groups > 0x7fffffffLL) return MSGL_ERR_SHAPE;
+  const int nct = nct_for(cols);
+  if (a.head_dim == 128) return launch_d<128>(p, nct, nw, stream);
+  if (a.head_dim == 256) return launch_d<256>(p, nct, nw, stream);
   return MSGL_ERR_HEAD_DIM;
 }
 

@@ -40,8 +40,8 @@ SIGNATURES = {
 
 MSGL_DTYPE_BF16 = 0
 MSGL_DTYPE_F16 = 1
-TUNE_DECODE_CHUNK = 0
-TUNE_SMALLQ_CHUNK = 1
+TUNE_SEGMENTS = 0
+TUNE_MIN_SEGMENT = 1
 TUNE_SMALLQ_MAXCOLS = 2
 TUNE_PREFILL_VARIANT = 3
 

@@ -23,17 +23,22 @@ def test_decode_group_sizes(gpu, n_q, n_kv):
     _check(wl, gpu, f"decode n_q={n_q} n_kv={n_kv}")
 
 
-@pytest.mark.parametrize("chunk", [32, 64, 96, 256, 4096])
-def test_decode_result_independent_of_chunking(gpu, chunk):
+@pytest.mark.parametrize("segments,min_seg", [(1, 64), (2, 64), (3, 128), (7, 64), (55, 64),
+                                              (4000, 64), (0, 0)])
+def test_decode_result_independent_of_the_split(gpu, segments, min_seg):
+    """Segment boundaries fall inside requests, on request boundaries, and (with one
+    segment) nowhere; the merged result must not depend on them."""
     from mini_sglang_amd_kernel import _lib
 
     wl = build_workload("t", "decode", seed=7, n_q=32, n_kv=8,
-                        kv_lens=[5, 100, 257, 1000, 2049, 31, 64], pool_factor=1.2)
-    _lib.set_tuning(_lib.TUNE_DECODE_CHUNK, chunk)
+                        kv_lens=[5, 100, 257, 1000, 2049, 31, 64, 0, 640], pool_factor=1.2)
+    _lib.set_tuning(_lib.TUNE_SEGMENTS, segments)
+    _lib.set_tuning(_lib.TUNE_MIN_SEGMENT, min_seg)
     try:
-        _check(wl, gpu, f"decode chunk={chunk}")
+        _check(wl, gpu, f"decode segments={segments} min_seg={min_seg}")
     finally:
-        _lib.set_tuning(_lib.TUNE_DECODE_CHUNK, 0)
+        _lib.set_tuning(_lib.TUNE_SEGMENTS, 0)
+        _lib.set_tuning(_lib.TUNE_MIN_SEGMENT, 0)
 
 
 def test_decode_empty_request_gives_zeros_and_page_size_one(gpu):

@@ -107,12 +107,14 @@ def test_splitk_route_ragged_q_and_chunking(gpu):
     wl = build_workload("t", "prefill", seed=310, n_q=8, n_kv=2,
                         kv_lens=[5, 100 + 8, 700 + 3, 64 + 16], extend_lens=[5, 8, 3, 16],
                         pool_factor=1.1, store_new=True, sliding_window_size=50)
-    for chunk in (32, 128, 0):
-        _lib.set_tuning(_lib.TUNE_SMALLQ_CHUNK, chunk)
+    for segments in (1, 5, 64, 0):
+        _lib.set_tuning(_lib.TUNE_SEGMENTS, segments)
+        _lib.set_tuning(_lib.TUNE_MIN_SEGMENT, 64)
         try:
-            _check(wl, gpu, f"split-K route ragged chunk={chunk}")
+            _check(wl, gpu, f"split-K route ragged segments={segments}")
         finally:
-            _lib.set_tuning(_lib.TUNE_SMALLQ_CHUNK, 0)
+            _lib.set_tuning(_lib.TUNE_SEGMENTS, 0)
+            _lib.set_tuning(_lib.TUNE_MIN_SEGMENT, 0)
 
 
 def test_both_routes_agree_and_decode_equals_prefill_qlen1(gpu):
