@@ -41,24 +41,34 @@ def log(*a):
 
 
 def time_steps(fn, steps: int, warmup: int):
-    """Per-step durations (ms) from HIP events recorded on torch's current stream, which is
-    the stream every operator launches on."""
+    """Time exactly `steps` back-to-back steps between two HIP events recorded on torch's
+    current stream (the stream every operator launches on), bracketed by device syncs.
+    A second pass brackets every step with its own event pair for the min / median; those
+    figures carry the event markers' own few microseconds."""
     import torch
 
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    loop_ms = e0.elapsed_time(e1)
     starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
     ends = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
-    t0 = time.perf_counter()
     for i in range(steps):
         starts[i].record()
         fn()
         ends[i].record()
     torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3
     per = [s.elapsed_time(e) for s, e in zip(starts, ends)]
-    return per, wall_ms
+    return loop_ms / steps, per, wall_ms
 
 
 def make_step(g):
@@ -131,8 +141,7 @@ def run_config(cfg: int, variant: str, steps: int, warmup: int, check: bool, cpu
     step = make_step(g)
     out = step()
     torch.cuda.synchronize()
-    per, wall_ms = time_steps(step, steps, warmup)
-    mean_ms = sum(per) / len(per)
+    mean_ms, per, wall_ms = time_steps(step, steps, warmup)
     med_ms = statistics.median(per)
     abytes = wl.attention_bytes()
     aflops = wl.attention_flops()

@@ -151,11 +151,13 @@ MSGL_API int msgl_paged_prefill_attention(const void* q, const void* k_cache, co
  *   MSGL_TUNE_MIN_SEGMENT    smallest segment length in tokens (multiple of 64)
  *   MSGL_TUNE_SMALLQ_MAXCOLS largest q_len*group routed to the split-K kernel
  *   MSGL_TUNE_PREFILL_VARIANT tiling of the MFMA kernel (0: 8 waves x 32 rows, 1: 4 x 64)
+ *   MSGL_TUNE_SPLITKV_WAVES  most waves (adjacent kv heads) per split-K workgroup: 1, 2, 4, 8
  */
 #define MSGL_TUNE_SEGMENTS 0
 #define MSGL_TUNE_MIN_SEGMENT 1
 #define MSGL_TUNE_SMALLQ_MAXCOLS 2
 #define MSGL_TUNE_PREFILL_VARIANT 3
+#define MSGL_TUNE_SPLITKV_WAVES 4
 MSGL_API int msgl_set_tuning(int32_t knob, int64_t value);
 
 #ifdef __cplusplus

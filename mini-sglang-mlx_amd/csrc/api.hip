@@ -71,6 +71,10 @@ const char* msgl_strerror(int code) {
 }
 
 int msgl_set_tuning(int32_t knob, int64_t value) {
+  if (knob == MSGL_TUNE_SPLITKV_WAVES) {
+    msgl::splitkv_set_max_waves((int)value);
+    return MSGL_OK;
+  }
   if (knob == MSGL_TUNE_PREFILL_VARIANT) {
     msgl::set_tile_variant((int)value);
     return MSGL_OK;

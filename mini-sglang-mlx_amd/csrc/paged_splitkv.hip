@@ -8,10 +8,14 @@
 //
 // Work decomposition
 //   The visible keys of all requests, in CSR order, form one token stream.  It is cut
-//   into `n_seg` equal segments (the count is chosen on the host so that all workgroups
-//   are resident at once: one round, no tail).  A workgroup owns one segment and NW
-//   adjacent kv heads, one wave64 per head; its waves walk the same tokens, so the
-//   workgroup touches NW*256-byte stretches of every slot row together.  A segment may
+//   into `n_seg` equal segments (the count is chosen on the host: one workgroup per CU,
+//   all resident at once, one round, no tail; the HBM system, not the CUs, is the limit).
+//   A workgroup owns one segment and `nwh` adjacent kv heads, one wave64 per head; all
+//   waves walk the same tokens, so the workgroup touches nwh*256-byte stretches of every
+//   slot row together.  A wave holds up to two tiles of 16 columns; shapes with more
+//   columns add a second wave per head (measured: a second wave re-reading the rows costs
+//   about as much as reading them from HBM, so columns stay in one wave when they fit).
+//   A segment may
 //   cross request boundaries: the wave finishes one request's share (writing bf16 output
 //   directly if it covered the whole request, otherwise a normalised fp32 partial + base-2
 //   LSE) and continues with the next.  splitkv_merge_kernel combines the partials.
@@ -57,7 +61,8 @@ struct SplitKvParams {
   int32_t* seg_info;    // [0] = segment length the attention kernel used
   int64_t k_stride0, v_stride0;
   int32_t batch, n_q, n_kv, group;
-  int32_t head_groups;  // n_kv / waves per workgroup
+  int32_t nwh;          // kv heads per workgroup
+  int32_t head_groups;  // n_kv / nwh
   int32_t n_seg, min_seg, cols, max_len_extend;
   int32_t is_cross, window;
   float scale_log2e;
@@ -154,12 +159,10 @@ struct KvTile {
   u32x4_t v[D / 128][8];  // [128-wide half of D][token j of the lane group]: raw V segments
 };
 
-// Two waves per SIMD where the register budget allows it (256 VGPRs each).
-template <int D, int NCT>
-constexpr int splitkv_min_waves() { return (D == 128 && NCT == 1) ? 2 : 1; }
-
+// NCT = tiles of 16 columns per wave, NW = waves per workgroup (launch bound only).  One
+// column tile at head dim 128 fits 256 VGPRs, so two such waves per SIMD can be resident.
 template <int D, int NCT, int NW>
-__global__ __launch_bounds__(64 * NW, (splitkv_min_waves<D, NCT>())) void splitkv_attention_kernel(SplitKvParams p) {
+__global__ __launch_bounds__(64 * NW, ((D == 128 && NCT == 1) ? 2 : 1)) void splitkv_attention_kernel(SplitKvParams p) {
   constexpr int KS = D / 32;   // k-steps of the QK product
   constexpr int VH = D / 128;  // 128-wide halves of D in the PV product
   const int lane = lane_id();
@@ -167,7 +170,10 @@ __global__ __launch_bounds__(64 * NW, (splitkv_min_waves<D, NCT>())) void splitk
   const int g = lane >> 4;
 
   const int seg = blockIdx.x / p.head_groups;
-  const int kvh = (blockIdx.x - seg * p.head_groups) * NW + (threadIdx.x >> 6);
+  const int wave = threadIdx.x >> 6;
+  const int cw = wave / p.nwh;  // which share of the columns this wave owns
+  const int ct0 = cw * NCT;     // first of its tiles of 16 columns
+  const int kvh = (blockIdx.x - seg * p.head_groups) * p.nwh + (wave - cw * p.nwh);
   int seg_len, total, cur_b, vs;
   if (!locate_segment(p, seg, &seg_len, &total, &cur_b, &vs)) return;
   if (blockIdx.x == 0 && threadIdx.x == 0) p.seg_info[0] = seg_len;
@@ -189,7 +195,7 @@ __global__ __launch_bounds__(64 * NW, (splitkv_min_waves<D, NCT>())) void splitk
     const int t_begin = r.lo + (vpos - vs);
     const int t_end = min(r.hi, t_begin + (seg_end - vpos));
     const bool whole = (t_begin == r.lo) && (t_end == r.hi);
-    if (t_begin == r.lo && kvh == 0 && lane == 0) p.req_vstart[cur_b] = vs;
+    if (t_begin == r.lo && kvh == 0 && ct0 == 0 && lane == 0) p.req_vstart[cur_b] = vs;
     const int ncols = r.q_len * p.group;
 
     // ---- Q operand and per-column visibility bounds --------------------------------
@@ -198,7 +204,7 @@ __global__ __launch_bounds__(64 * NW, (splitkv_min_waves<D, NCT>())) void splitk
     int all_lo = 0, all_hi = 0x7fffffff;  // tile is mask-free iff inside [all_lo, all_hi]
 #pragma unroll
     for (int ct = 0; ct < NCT; ++ct) {
-      const int col = ct * 16 + t16;
+      const int col = (ct0 + ct) * 16 + t16;
       const bool valid = col < ncols;
       const int qi = valid ? col / p.group : 0;
       const int hh = valid ? col - qi * p.group : 0;
@@ -378,7 +384,7 @@ __global__ __launch_bounds__(64 * NW, (splitkv_min_waves<D, NCT>())) void splitk
       l += __shfl_xor(l, 16, kWave);
       l += __shfl_xor(l, 32, kWave);
       const float inv = (l > 0.f) ? 1.0f / l : 0.f;
-      const int col = ct * 16 + t16;
+      const int col = (ct0 + ct) * 16 + t16;
       if (col >= ncols) continue;
       const int qi = col / p.group;
       const int hh = col - qi * p.group;
@@ -493,61 +499,47 @@ __global__ __launch_bounds__(64) void splitkv_merge_kernel(SplitKvParams p) {
     *reinterpret_cast<uint32_t*>(orow + e) = pack_bf16x2(acc[e] * inv, acc[e + 1] * inv);
 }
 
-int waves_per_group(int64_t n_kv) { return (n_kv % 4 == 0) ? 4 : (n_kv % 2 == 0) ? 2 : 1; }
+int nct_for(int64_t cols) { return (int)((cols + 15) / 16); }
 
-// Workgroups of a kernel variant that one GPU holds at the same time.
-template <typename K>
-int resident_blocks(K kernel, int block_threads, std::atomic<int>& cache) {
+std::atomic<int> g_max_waves{4};
+int heads_per_group(int64_t n_kv) {
+  const int cap = g_max_waves.load();
+  if (cap >= 8 && n_kv % 8 == 0) return 8;
+  if (cap >= 4 && n_kv % 4 == 0) return 4;
+  return (cap >= 2 && n_kv % 2 == 0) ? 2 : 1;
+}
+
+int device_cus() {
+  static std::atomic<int> cache{0};
   int v = cache.load();
   if (v > 0) return v;
-  int dev = 0, cus = 0, per_cu = 0;
+  int dev = 0, cus = 0;
   if (hipGetDevice(&dev) != hipSuccess ||
       hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
-      hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, block_threads, 0) != hipSuccess ||
-      cus <= 0 || per_cu <= 0) {
+      cus <= 0) {
     (void)hipGetLastError();
-    return 512;  // MI355X: 256 CUs x 2
+    return 256;  // MI355X
   }
-  v = cus * per_cu;
-  cache.store(v);
-  return v;
+  cache.store(cus);
+  return cus;
 }
 
 template <int D, int NCT, int NW>
-int resident_for() {
-  static std::atomic<int> cache{0};
-  return resident_blocks(splitkv_attention_kernel<D, NCT, NW>, 64 * NW, cache);
+void launch_attn(const SplitKvParams& p, hipStream_t stream) {
+  hipLaunchKernelGGL((splitkv_attention_kernel<D, NCT, NW>),
+                     dim3((unsigned)(p.n_seg * p.head_groups)), dim3(64 * NW), 0, stream, p);
 }
 
-template <int D, int NW>
-int resident_dw(int nct) {
-  switch (nct) {
-    case 1: return resident_for<D, 1, NW>();
-    case 2: return resident_for<D, 2, NW>();
-    case 3: return resident_for<D, 3, NW>();
-    default: return resident_for<D, 4, NW>();
-  }
-}
-
-int resident_any(int64_t head_dim, int nct, int nw) {
-  if (head_dim == 128) {
-    if (nw == 4) return resident_dw<128, 4>(nct);
-    if (nw == 2) return resident_dw<128, 2>(nct);
-    return resident_dw<128, 1>(nct);
-  }
-  if (nw == 4) return resident_dw<256, 4>(nct);
-  if (nw == 2) return resident_dw<256, 2>(nct);
-  return resident_dw<256, 1>(nct);
-}
-
-template <int D, int NW>
-int launch_dw(const SplitKvParams& p, int nct, hipStream_t stream) {
-  const dim3 grid((unsigned)(p.n_seg * p.head_groups)), block(64 * NW);
-  switch (nct) {
-    case 1: hipLaunchKernelGGL((splitkv_attention_kernel<D, 1, NW>), grid, block, 0, stream, p); break;
-    case 2: hipLaunchKernelGGL((splitkv_attention_kernel<D, 2, NW>), grid, block, 0, stream, p); break;
-    case 3: hipLaunchKernelGGL((splitkv_attention_kernel<D, 3, NW>), grid, block, 0, stream, p); break;
-    case 4: hipLaunchKernelGGL((splitkv_attention_kernel<D, 4, NW>), grid, block, 0, stream, p); break;
+template <int D, int NCT>
+int launch_dn(const SplitKvParams& p, int waves, hipStream_t stream) {
+  switch (waves) {
+    case 1: launch_attn<D, NCT, 1>(p, stream); break;
+    case 2: launch_attn<D, NCT, 2>(p, stream); break;
+    case 4: launch_attn<D, NCT, 4>(p, stream); break;
+    case 8:
+      if constexpr (D == 128 && NCT == 1) launch_attn<D, NCT, 8>(p, stream);
+      else return MSGL_ERR_SHAPE;
+      break;
     default: return MSGL_ERR_SHAPE;
   }
   int rc = check_launch();
@@ -557,23 +549,46 @@ int launch_dw(const SplitKvParams& p, int nct, hipStream_t stream) {
   return check_launch();
 }
 
-template <int D>
-int launch_d(const SplitKvParams& p, int nct, int nw, hipStream_t stream) {
-  if (nw == 4) return launch_dw<D, 4>(p, nct, stream);
-  if (nw == 2) return launch_dw<D, 2>(p, nct, stream);
-  return launch_dw<D, 1>(p, nct, stream);
+// How a shape's column tiles map onto waves: tiles per wave and waves per kv head.
+struct ColSplit { int nct_wave; int col_waves; };
+ColSplit col_split(int nct, int64_t head_dim) {
+  if (head_dim != 128) return ColSplit{1, nct};  // two tiles at head dim 256 would spill
+  return nct <= 2 ? ColSplit{nct, 1} : ColSplit{2, 2};
 }
 
-int nct_for(int64_t cols) { return (int)((cols + 15) / 16); }
+template <int D>
+int launch_d(const SplitKvParams& p, int nct, hipStream_t stream) {
+  const ColSplit cs = col_split(nct, D);
+  const int waves = p.nwh * cs.col_waves;
+  if (cs.nct_wave == 1) return launch_dn<D, 1>(p, waves, stream);
+  if constexpr (D == 128) return launch_dn<D, 2>(p, waves, stream);
+  return MSGL_ERR_SHAPE;
+}
 
 }  // namespace
 
+void splitkv_set_max_waves(int v) { g_max_waves.store(v); }
+
+// kv heads per workgroup for this shape: up to 4, halved when a second wave per head is
+// needed for the columns (a workgroup of the wide variants holds at most 4 waves: they
+// need more than 256 VGPRs, one wave per SIMD)
+static int nwh_for(int64_t n_kv, int nct, int64_t head_dim) {
+  int nwh = heads_per_group(n_kv);
+  const int col_waves = col_split(nct, head_dim).col_waves;
+  const int max_waves = (nct == 1 && head_dim == 128) ? 8 : 4;
+  while (nwh * col_waves > max_waves && nwh > 1) nwh /= 2;
+  return nwh;
+}
+
 int splitkv_default_segments(int64_t total_kv, int64_t n_kv, int64_t head_dim, int64_t cols,
                              int32_t min_seg) {
-  const int nw = waves_per_group(n_kv);
-  const int64_t head_groups = n_kv / nw;
-  const int resident = resident_any(head_dim, nct_for(cols), nw);
-  int64_t n_seg = resident / head_groups;  // one resident round
+  const int nct = nct_for(cols);
+  const int nwh = nwh_for(n_kv, nct, head_dim);
+  const int waves = nwh * col_split(nct, head_dim).col_waves;
+  const int64_t head_groups = n_kv / nwh;
+  // one workgroup per CU; small workgroups are doubled up until a CU holds four waves
+  const int64_t blocks = (int64_t)device_cus() * (waves >= 4 ? 1 : 4 / waves);
+  int64_t n_seg = blocks / head_groups;
   const int64_t by_len = (total_kv + min_seg - 1) / min_seg;
   if (n_seg > by_len) n_seg = by_len;
   if (n_seg < 1) n_seg = 1;
@@ -597,7 +612,8 @@ int launch_splitkv(const SplitKvArgs& a, hipStream_t stream) {
     return MSGL_ERR_SHAPE;
   if (a.batch * a.max_len_extend > 0x7fffffffLL || a.total_kv > 0x7fffffffLL) return MSGL_ERR_SHAPE;
   if (a.batch == 0) return MSGL_OK;
-  const int nw = waves_per_group(a.n_kv);
+  const int nct = nct_for(cols);
+  const int nwh = nwh_for(a.n_kv, nct, a.head_dim);
 
   SplitKvParams p;
   p.q = static_cast<const uint16_t*>(a.q);
@@ -621,7 +637,8 @@ int launch_splitkv(const SplitKvArgs& a, hipStream_t stream) {
   p.n_q = (int32_t)a.n_q;
   p.n_kv = (int32_t)a.n_kv;
   p.group = (int32_t)group;
-  p.head_groups = (int32_t)(a.n_kv / nw);
+  p.nwh = nwh;
+  p.head_groups = (int32_t)(a.n_kv / nwh);
   p.n_seg = a.n_seg;
   p.min_seg = a.min_seg;
   p.max_len_extend = a.max_len_extend;
@@ -629,9 +646,8 @@ int launch_splitkv(const SplitKvArgs& a, hipStream_t stream) {
   p.window = a.window;
   p.scale_log2e = a.sm_scale * kLog2e;
   if ((int64_t)p.n_seg * p.head_groups > 0x7fffffffLL) return MSGL_ERR_SHAPE;
-  const int nct = nct_for(cols);
-  if (a.head_dim == 128) return launch_d<128>(p, nct, nw, stream);
-  if (a.head_dim == 256) return launch_d<256>(p, nct, nw, stream);
+  if (a.head_dim == 128) return launch_d<128>(p, nct, stream);
+  if (a.head_dim == 256) return launch_d<256>(p, nct, stream);
   return MSGL_ERR_HEAD_DIM;
 }
 

@@ -44,6 +44,7 @@ TUNE_SEGMENTS = 0
 TUNE_MIN_SEGMENT = 1
 TUNE_SMALLQ_MAXCOLS = 2
 TUNE_PREFILL_VARIANT = 3
+TUNE_SPLITKV_WAVES = 4
 
 _lib = None
 
