@@ -1,0 +1,118 @@
+"""The five benchmark shapes at FULL size on the GPU.
+
+Parity against the CPU oracle on the same seeded inputs (all requests where the oracle
+finishes in seconds, the shortest requests otherwise), KV-pool bit-exactness after the
+store, and size-independent properties at full size: independence of the split, one extend
+== two chunked extends, decode(L) == extend(q_len 1)."""
+import pytest
+import torch
+
+import oracle
+from _gpu_util import run_gpu, run_oracle
+from _util import assert_close_bf16
+from mini_sglang_amd.workloads import config_workload
+
+pytestmark = pytest.mark.gpu
+
+
+def _shortest(wl, n):
+    order = sorted(range(wl.batch), key=lambda b: wl.kv_lens[b])
+    return sorted(order[:n])
+
+
+def test_cfg1_small_decode_full_oracle(gpu):
+    wl = config_workload(1)
+    assert wl.kv_lens == [37, 128, 500, 1023] and wl.k_cache.shape[0] == 512 * 16
+    got, _ = run_gpu(wl, gpu)
+    want, _ = run_oracle(wl)
+    assert_close_bf16(got, want, "cfg1")
+
+
+def test_cfg2_decode_batch64_full_oracle(gpu):
+    print("cfg2 build", flush=True)
+    wl = config_workload(2)
+    assert wl.batch == 64 and min(wl.kv_lens) >= 1024 and max(wl.kv_lens) <= 8192
+    got, _ = run_gpu(wl, gpu)
+    print("cfg2 oracle", flush=True)
+    want, _ = run_oracle(wl, precision="f32")
+    assert_close_bf16(got, want, "cfg2")
+
+
+def test_cfg3_chunked_extend_with_store(gpu):
+    from mini_sglang_amd_kernel import paged_prefill_attention, store_kv_cache
+
+    print("cfg3 build", flush=True)
+    wl = config_workload(3)
+    assert wl.batch == 8 and wl.extend_lens == [512] * 8
+    got, g = run_gpu(wl, gpu)
+    assert torch.isfinite(got.float()).all()
+    # pools after the store: bit-exact against the oracle's row scatter
+    ref = wl.clone_pools()
+    oracle.store_kv_cache(ref.k_cache, ref.v_cache, ref.out_loc, ref.new_k, ref.new_v)
+    assert torch.equal(g.k_cache.cpu().view(torch.int16), ref.k_cache.view(torch.int16))
+    assert torch.equal(g.v_cache.cpu().view(torch.int16), ref.v_cache.view(torch.int16))
+    # oracle on the two shortest requests (all 512 rows, all heads)
+    reqs = _shortest(wl, 2)
+    print(f"cfg3 oracle on requests {reqs}", flush=True)
+    sub = wl.select(reqs)
+    want, _ = run_oracle(sub, precision="f32")
+    qo = wl.qo_indptr.tolist()
+    rows = torch.cat([torch.arange(qo[b], qo[b + 1]) for b in reqs])
+    assert_close_bf16(got[rows], want, "cfg3 sampled requests")
+    # full size, no oracle: one 512-token extend == a 256-token extend then another on
+    # prefix + 256 (the stored pool already holds all 512 new rows)
+    print("cfg3 chunked-extend property", flush=True)
+    halves = []
+    for part in (0, 1):
+        ext = [256] * wl.batch
+        kv_lens = [p + 256 * (part + 1) for p in wl.prefixes]
+        ip = wl.kv_indptr.tolist()
+        idx = torch.cat([wl.kv_indices[ip[b]:ip[b] + kv_lens[b]] for b in range(wl.batch)])
+        qrows = torch.cat([torch.arange(qo[b] + 256 * part, qo[b] + 256 * (part + 1))
+                           for b in range(wl.batch)])
+        kvp = torch.cumsum(torch.tensor([0] + kv_lens), 0).to(torch.int32)
+        qop = torch.cumsum(torch.tensor([0] + ext), 0).to(torch.int32)
+        pre = torch.tensor([p + 256 * part for p in wl.prefixes], dtype=torch.int32)
+        out = paged_prefill_attention(g.q[qrows.to(gpu)], g.k_cache, g.v_cache, qop.to(gpu),
+                                      kvp.to(gpu), idx.to(gpu), pre.to(gpu), g.sm_scale, 256)
+        halves.append((qrows, out.cpu()))
+    torch.cuda.synchronize()
+    for qrows, out in halves:
+        assert_close_bf16(out, got[qrows].float(), "cfg3 chunked extend", max_tol=8e-3, mean_tol=4e-4)
+
+
+def test_cfg4_long_context_decode_split_and_sampled_oracle(gpu):
+    from mini_sglang_amd_kernel import _lib
+
+    print("cfg4 build", flush=True)
+    wl = config_workload(4, pool_device=gpu)
+    assert wl.batch == 16 and min(wl.kv_lens) >= 32768 and max(wl.kv_lens) <= 131072
+    got, g = run_gpu(wl, gpu)
+    assert torch.isfinite(got.float()).all()
+    # the merged result must not depend on where the stream is cut
+    for segments in (16, 509):
+        print(f"cfg4 segments={segments}", flush=True)
+        _lib.set_tuning(_lib.TUNE_SEGMENTS, segments)
+        try:
+            other, _ = run_gpu(wl, gpu)
+        finally:
+            _lib.set_tuning(_lib.TUNE_SEGMENTS, 0)
+        assert_close_bf16(other, got.float(), f"cfg4 split invariance ({segments})",
+                          max_tol=4e-3, mean_tol=2e-4)
+    reqs = _shortest(wl, 2)
+    print(f"cfg4 oracle on requests {reqs}", flush=True)
+    sub = wl.select(reqs).to("cpu")
+    want, _ = run_oracle(sub, precision="f32")
+    assert_close_bf16(got[reqs], want, "cfg4 sampled requests")
+
+
+@pytest.mark.parametrize("variant", ["", "window"])
+def test_cfg5_speculative_verify_full_oracle(gpu, variant):
+    print(f"cfg5 {variant} build", flush=True)
+    wl = config_workload(5, variant=variant)
+    assert wl.batch == 32 and wl.extend_lens == [8] * 32
+    assert wl.sliding_window_size == (1024 if variant else 0)
+    got, _ = run_gpu(wl, gpu)
+    print("cfg5 oracle", flush=True)
+    want, _ = run_oracle(wl, precision="f32")
+    assert_close_bf16(got, want, f"cfg5 {variant}")
