@@ -176,12 +176,16 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
   const uint16_t* kbase = p.k_cache + (int64_t)kvh * D + c * 8;
   const uint16_t* vbase = p.v_cache + (int64_t)kvh * D + c * 8;
   u32x4_t kr[KPT], vr[KPT];
-  auto stage_load = [&](int tb) {
+  int32_t slot[KPT];  // slot ids of the NEXT tile to load, fetched one tile ahead
+  auto slot_load = [&](int tb) {
+#pragma unroll
+    for (int i = 0; i < KPT; ++i) slot[i] = idx_base[min(tb + key0 + i, kn - 1)];
+  };
+  auto stage_load = [&]() {
 #pragma unroll
     for (int i = 0; i < KPT; ++i) {
-      const int64_t slot = idx_base[min(tb + key0 + i, kn - 1)];
-      kr[i] = ld_global_b128(kbase + slot * p.k_stride0);
-      vr[i] = ld_global_b128(vbase + slot * p.v_stride0);
+      kr[i] = ld_global_b128(kbase + (int64_t)slot[i] * p.k_stride0);
+      vr[i] = ld_global_b128(vbase + (int64_t)slot[i] * p.v_stride0);
     }
   };
   auto stage_store = [&](int buf) {
@@ -305,18 +309,24 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
   };
 
   // ---- main loop ---------------------------------------------------------------------
+  // Every load and LDS store below is unconditional (tiles past the end clamp to the last
+  // key and are never read), so the loop body has one fixed sequence of memory operations:
+  // the next tile's rows are in flight during the whole compute phase and the slot ids of
+  // the tile after it were fetched a full iteration earlier.
   if (n_tiles > 0) {
-    stage_load(k_lo);
+    slot_load(k_lo);
+    stage_load();
+    slot_load(k_lo + kBN);
     stage_store(0);
-  }
-  __syncthreads();
-  for (int t = 0; t < n_tiles; ++t) {
-    const int tb = k_lo + t * kBN;
-    const bool more = (t + 1 < n_tiles);
-    if (more) stage_load(tb + kBN);
-    if (tb <= w_hi_max && tb + kBN - 1 >= w_lo_min) compute_tile(t & 1, tb);
-    if (more) stage_store((t + 1) & 1);
     __syncthreads();
+    for (int t = 0; t < n_tiles; ++t) {
+      const int tb = k_lo + t * kBN;
+      stage_load();                // rows of tile t+1
+      slot_load(tb + 2 * kBN);     // slot ids of tile t+2
+      if (tb <= w_hi_max && tb + kBN - 1 >= w_lo_min) compute_tile(t & 1, tb);
+      stage_store((t + 1) & 1);
+      __syncthreads();
+    }
   }
 
   // ---- epilogue: normalise, un-permute through LDS, store whole rows -----------------
