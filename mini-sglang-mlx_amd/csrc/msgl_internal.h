@@ -57,7 +57,7 @@ struct PrefillArgs {
   const int32_t* kv_indices;
   const int32_t* prefix_lens;
   void* out;
-  int64_t batch, total_q, total_kv, n_q, n_kv, head_dim;
+  int64_t batch, total_q, total_kv, n_q, n_kv, head_dim, num_slots;
   int64_t k_stride0, v_stride0;  // elements
   float sm_scale;
   int32_t max_len_extend;

@@ -23,12 +23,19 @@
 //
 // Algorithmic flops: 4 * D per visible (query, key) pair and q head (QK^T + PV).
 #include <atomic>
+#include <type_traits>
 
 #include "msgl_device.h"
 #include "msgl_internal.h"
 
 namespace msgl {
 namespace {
+
+#ifdef MSGL_PROFILE_PHASES
+#define MSGL_TICK(i) do { const long long t_ = clock64(); prof_acc[i] += t_ - prof_t; prof_t = t_; } while (0)
+#else
+#define MSGL_TICK(i) do { } while (0)
+#endif
 
 struct PrefillParams {
   const uint16_t* q;
@@ -44,6 +51,9 @@ struct PrefillParams {
   int32_t n_qblk, n_pairs;  // q blocks per (request, kv head); batch * n_kv
   int32_t max_len_extend, is_cross, window;
   float scale_log2e;
+#ifdef MSGL_PROFILE_PHASES
+  long long* prof;  // [blocks][8] cycle totals of wave 0
+#endif
 };
 
 constexpr int kBN = 64;  // keys per tile
@@ -60,11 +70,14 @@ struct Smem {
   static constexpr int STAGE_BYTES = K_BYTES + V_BYTES;
   static constexpr int OROW = D + 8;
   static constexpr int O_BYTES = ROWS * OROW * 2;
-  static constexpr int TOTAL = (2 * STAGE_BYTES > O_BYTES) ? 2 * STAGE_BYTES : O_BYTES;
+  static constexpr int STAGES = 4;
+  static constexpr int TOTAL = (STAGES * STAGE_BYTES > O_BYTES) ? STAGES * STAGE_BYTES : O_BYTES;
 };
 
 // RT = 32-row tiles per wave, NW = waves per workgroup; the workgroup covers NW*RT*32 rows.
-template <int D, int RT, int NW>
+// WIDE: pool byte offsets need 64 bits (pool of 4 GiB or more); otherwise a row's offset
+// is one 32-bit multiply instead of a 64-bit multiply-add per load.
+template <int D, int RT, int NW, bool WIDE>
 __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) {
   static_assert(D == 128, "tile kernel is instantiated for head_dim 128");
   constexpr int kRows = NW * RT * 32;
@@ -83,14 +96,29 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
 
   // ---- block -> (request, kv head, q block).  Consecutive block ids go to different
   // XCDs; the q blocks of one (request, kv head) share an XCD (and its L2) and are
-  // issued back to back, heaviest (latest rows) first.
+  // issued back to back, heaviest (latest rows) first.  Requests are taken in order of
+  // decreasing kv length (longest-processing-time-first: the dispatcher hands out blocks
+  // in id order, so long requests start first and short ones fill the tail); each block
+  // finds "the request of rank r" itself from kv_indptr, the host never sees the lengths.
   const int xcd = blockIdx.x & 7;
   const int seq = blockIdx.x >> 3;
   const int pair = (seq / p.n_qblk) * 8 + xcd;
   if (pair >= p.n_pairs) return;
   const int qblk = p.n_qblk - 1 - (seq % p.n_qblk);
-  const int b = pair / p.n_kv;
-  const int kvh = pair - b * p.n_kv;
+  const int want_rank = pair / p.n_kv;
+  const int kvh = pair - want_rank * p.n_kv;
+  __shared__ int ranked_request;
+  for (int i = tid; i < p.batch; i += NW * 64) {
+    const int len_i = p.kv_indptr[i + 1] - p.kv_indptr[i];
+    int rank = 0;
+    for (int j = 0; j < p.batch; ++j) {
+      const int len_j = p.kv_indptr[j + 1] - p.kv_indptr[j];
+      rank += (len_j > len_i) || (len_j == len_i && j < i);
+    }
+    if (rank == want_rank) ranked_request = i;
+  }
+  __syncthreads();
+  const int b = ranked_request;
 
   const int q_start = p.qo_indptr[b];
   const int q_len = min(p.qo_indptr[b + 1] - q_start, p.max_len_extend);
@@ -173,8 +201,14 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
   const int key0 = kg * KPT;
   const int pos0 = (key0 & ~12) | ((key0 & 4) << 1) | ((key0 & 8) >> 1);  // key bits 2 <-> 3
   const int32_t* idx_base = p.kv_indices + kv_start;
-  const uint16_t* kbase = p.k_cache + (int64_t)kvh * D + c * 8;
-  const uint16_t* vbase = p.v_cache + (int64_t)kvh * D + c * 8;
+  const unsigned char* kbase = reinterpret_cast<const unsigned char*>(p.k_cache + (int64_t)kvh * D + c * 8);
+  const unsigned char* vbase = reinterpret_cast<const unsigned char*>(p.v_cache + (int64_t)kvh * D + c * 8);
+  const uint32_t k_row_bytes = (uint32_t)p.k_stride0 * 2u;
+  const uint32_t v_row_bytes = (uint32_t)p.v_stride0 * 2u;
+  auto row_offset = [](uint32_t slot_id, uint32_t row_bytes) -> uint64_t {
+    if constexpr (WIDE) return (uint64_t)slot_id * row_bytes;
+    else return (uint64_t)(slot_id * row_bytes);
+  };
   u32x4_t kr[KPT], vr[KPT];
   int32_t slot[KPT];  // slot ids of the NEXT tile to load, fetched one tile ahead
   auto slot_load = [&](int tb) {
@@ -184,8 +218,8 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
   auto stage_load = [&]() {
 #pragma unroll
     for (int i = 0; i < KPT; ++i) {
-      kr[i] = ld_global_b128(kbase + (int64_t)slot[i] * p.k_stride0);
-      vr[i] = ld_global_b128(vbase + (int64_t)slot[i] * p.v_stride0);
+      kr[i] = ld_global_b128(kbase + row_offset((uint32_t)slot[i], k_row_bytes));
+      vr[i] = ld_global_b128(vbase + row_offset((uint32_t)slot[i], v_row_bytes));
     }
   };
   auto stage_store = [&](int buf) {
@@ -212,121 +246,277 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
     }
   };
 
-  auto compute_tile = [&](int buf, int tb) {
-    const unsigned char* ks = smem + buf * S::STAGE_BYTES;
-    const unsigned char* vs = ks + S::K_BYTES;
-    // S^T[key][row]: lane holds key = tb + 32kt + 8(i/4) + 4h + i%4, row = 32rt + c32
-    f32x16_t s[2][RT];
+  // ---- the three pieces of one half tile (32 keys) --------------------------------------
+  struct Scores {
+    f32x16_t s[RT];  // S^T[key][row]: key = base + 8(i/4) + 4h + i%4, row = 32rt + c32
+  };
+  auto qk_half = [&](int buf, int kt, Scores& sc) {
+    const unsigned char* ks = smem + buf * S::STAGE_BYTES + (kt * 32 + c32) * S::KROW * 2 + h * 16;
 #pragma unroll
-    for (int kt = 0; kt < 2; ++kt)
+    for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-      for (int rt = 0; rt < RT; ++rt)
+      for (int i = 0; i < 16; ++i) sc.s[rt][i] = 0.f;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) s[kt][rt][i] = 0.f;
+    for (int kstep = 0; kstep < KSTEPS; ++kstep) {
+      const bf16x8_t a = as_bf16x8(*reinterpret_cast<const u32x4_t*>(ks + kstep * 32));
 #pragma unroll
-    for (int kstep = 0; kstep < KSTEPS; ++kstep)
-#pragma unroll
-      for (int kt = 0; kt < 2; ++kt) {
-        const bf16x8_t a = as_bf16x8(*reinterpret_cast<const u32x4_t*>(
-            ks + ((kt * 32 + c32) * S::KROW + kstep * 16 + h * 8) * 2));
-#pragma unroll
-        for (int rt = 0; rt < RT; ++rt) s[kt][rt] = mfma_32x32x16(a, qreg[rt][kstep], s[kt][rt]);
-      }
-
-    const bool need_mask = (tb < w_lo_max) || (tb + kBN - 1 > w_hi_min);
-    bf16x8_t pb[RT][4];
+      for (int rt = 0; rt < RT; ++rt) sc.s[rt] = mfma_32x32x16(a, qreg[rt][kstep], sc.s[rt]);
+    }
+  };
+  // Online softmax step over 32 keys starting at `base`.  MASKED halves scale and mask
+  // explicitly; interior halves keep raw scores and fold the scale into the exp2 argument
+  // (max commutes with a positive scale).
+  auto softmax_half = [&](Scores& sc, int base, auto masked_tag, bf16x8_t (&pb)[RT][2],
+                          float (&alpha)[RT]) {
+    constexpr bool MASKED = decltype(masked_tag)::value;
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
-      if (need_mask) {
+      if constexpr (MASKED) {
 #pragma unroll
-        for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) {
-            const int key = tb + kt * 32 + 8 * (i >> 2) + 4 * h + (i & 3);
-            const float x = s[kt][rt][i] * p.scale_log2e;
-            s[kt][rt][i] = (key < row_lo[rt] || key > row_hi[rt]) ? kNegInf : x;
-          }
-      }
-      float mx = kNegInf;
-#pragma unroll
-      for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[kt][rt][i]);
-      // unmasked tiles keep raw scores: max commutes with a non-negative scale
-      if (!need_mask) {
-        if (p.scale_log2e < 0.f) {
-          mx = -kNegInf;
-#pragma unroll
-          for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) mx = fminf(mx, s[kt][rt][i]);
+        for (int i = 0; i < 16; ++i) {
+          const int key = base + 8 * (i >> 2) + 4 * h + (i & 3);
+          const float x = sc.s[rt][i] * p.scale_log2e;
+          sc.s[rt][i] = (key < row_lo[rt] || key > row_hi[rt]) ? kNegInf : x;
         }
-        mx *= p.scale_log2e;
       }
+      float mx = fmaxf(sc.s[rt][0], sc.s[rt][1]);
+#pragma unroll
+      for (int i = 2; i < 16; ++i) mx = fmaxf(mx, sc.s[rt][i]);
+      if constexpr (!MASKED) mx *= p.scale_log2e;
       mx = wave_max_xor(mx, 32);
       const float m_old = m_run[rt];
       const float m_new = fmaxf(m_old, mx);
       const float m_use = (m_new - m_old > kLazy) ? m_new : m_old;
       const float m_safe = (m_use == kNegInf) ? 0.f : m_use;
-      const float alpha = fast_exp2(m_old - m_safe);
+      alpha[rt] = fast_exp2(m_old - m_safe);
       m_run[rt] = m_use;
-      const float mul = need_mask ? 1.0f : p.scale_log2e;
+      const float mul = MASKED ? 1.0f : p.scale_log2e;
       float psum = 0.f;
 #pragma unroll
-      for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const float e = fast_exp2(__builtin_fmaf(s[kt][rt][i], mul, -m_safe));
-          s[kt][rt][i] = e;
-          psum += e;
-        }
-      l_run[rt] = l_run[rt] * alpha + psum;
-      if (__any(alpha != 1.0f)) {
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) oacc[dt][rt][i] *= alpha;
+      for (int i = 0; i < 16; ++i) {
+        const float e = fast_exp2(__builtin_fmaf(sc.s[rt][i], mul, -m_safe));
+        sc.s[rt][i] = e;
+        psum += e;
       }
+      l_run[rt] = l_run[rt] * alpha[rt] + psum;
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
+      for (int u = 0; u < 2; ++u) {
         u32x4_t pk;
 #pragma unroll
         for (int j = 0; j < 4; ++j)
-          pk[j] = pack_bf16x2(s[u >> 1][rt][8 * (u & 1) + 2 * j], s[u >> 1][rt][8 * (u & 1) + 2 * j + 1]);
+          pk[j] = pack_bf16x2(sc.s[rt][8 * u + 2 * j], sc.s[rt][8 * u + 2 * j + 1]);
         pb[rt][u] = as_bf16x8(pk);
       }
     }
-    // O^T[dim row][row] += V^T * P^T ; k-step u covers key positions 16u .. 16u+15
+  };
+  // O^T[dim row][row] += V^T * P^T over key positions 32kt .. 32kt+31 (two k-steps of 16)
+  auto pv_half = [&](int buf, int kt, const bf16x8_t (&pb)[RT][2]) {
+    const unsigned char* vs =
+        smem + buf * S::STAGE_BYTES + S::K_BYTES + c32 * S::VROW * 2 + (32 * kt + 8 * h) * 2;
 #pragma unroll
-    for (int u = 0; u < 4; ++u)
+    for (int u = 0; u < 2; ++u)
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) {
-        const bf16x8_t a = as_bf16x8(*reinterpret_cast<const u32x4_t*>(
-            vs + ((dt * 32 + c32) * S::VROW + 16 * u + 8 * h) * 2));
+        const bf16x8_t a = as_bf16x8(
+            *reinterpret_cast<const u32x4_t*>(vs + dt * 32 * S::VROW * 2 + u * 32));
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) oacc[dt][rt] = mfma_32x32x16(a, pb[rt][u], oacc[dt][rt]);
       }
   };
+  // O *= alpha where some row's lazy max moved (rare)
+  auto rescale = [&](const float (&alpha)[RT]) {
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      if (__any(alpha[rt] != 1.0f)) {
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) oacc[dt][rt][i] *= alpha[rt];
+      }
+    }
+  };
+  // One pipeline step over half tiles i-1, i, i+1: the matrix pipe computes the scores of
+  // half i+1 and adds P V of half i-1 while the VALU turns the scores of half i into P.
+  // The three pieces are independent.  The step is cut into four slices, each holding a
+  // quarter of the MFMAs (two K operands, two V operands) and a quarter of the softmax, with
+  // a scheduling barrier between slices: inside a slice the compiler interleaves MFMA, LDS
+  // reads and VALU freely, across slices nothing moves, which bounds operand live ranges.
+  // `mul` is the factor still to be applied to the scores: the softmax scale on interior
+  // halves (raw scores; max commutes with a positive scale), 1 on halves that apply_mask
+  // already scaled.
+  auto fused_half = [&](Scores& cur, float mul, Scores& nxt, int k_buf, int k_kt, int v_buf,
+                        int v_kt, const bf16x8_t (&pb_prev)[RT][2], bf16x8_t (&pb_cur)[RT][2],
+                        float (&alpha_cur)[RT]) {
+    const unsigned char* ks =
+        smem + k_buf * S::STAGE_BYTES + (k_kt * 32 + c32) * S::KROW * 2 + h * 16;
+    const unsigned char* vs =
+        smem + v_buf * S::STAGE_BYTES + S::K_BYTES + c32 * S::VROW * 2 + (32 * v_kt + 8 * h) * 2;
+    auto mfma_slice = [&](int sl) {
+      // alternate the two products: consecutive score MFMAs extend the same accumulator
+      // chain, the P V ones go to different accumulators
+      const int u = sl >> 1;
+#pragma unroll
+      for (int e = 0; e < 2; ++e) {
+        const int kstep = 2 * sl + e;
+        const bf16x8_t a = as_bf16x8(*reinterpret_cast<const u32x4_t*>(ks + kstep * 32));
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) nxt.s[rt] = mfma_32x32x16(a, qreg[rt][kstep], nxt.s[rt]);
+        const int dt = 2 * (sl & 1) + e;
+        const bf16x8_t b = as_bf16x8(
+            *reinterpret_cast<const u32x4_t*>(vs + dt * 32 * S::VROW * 2 + u * 32));
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) oacc[dt][rt] = mfma_32x32x16(b, pb_prev[rt][u], oacc[dt][rt]);
+      }
+    };
+    float m_safe[RT], psum[RT];
+    auto exp_slice = [&](int first) {  // elements first .. first+7
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int i = first; i < first + 8; ++i) {
+          const float e = fast_exp2(__builtin_fmaf(cur.s[rt][i], mul, -m_safe[rt]));
+          cur.s[rt][i] = e;
+          psum[rt] += e;
+        }
+    };
+    auto pack_slice = [&](int u) {
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        u32x4_t pk;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          pk[j] = pack_bf16x2(cur.s[rt][8 * u + 2 * j], cur.s[rt][8 * u + 2 * j + 1]);
+        pb_cur[rt][u] = as_bf16x8(pk);
+      }
+    };
+    // slice 0: row max, lazy-max decision
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) nxt.s[rt][i] = 0.f;
+    mfma_slice(0);
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      float mx = fmaxf(cur.s[rt][0], cur.s[rt][1]);
+#pragma unroll
+      for (int i = 2; i < 16; ++i) mx = fmaxf(mx, cur.s[rt][i]);
+      mx = wave_max_xor(mx * mul, 32);
+      const float m_old = m_run[rt];
+      const float m_new = fmaxf(m_old, mx);
+      const float m_use = (m_new - m_old > kLazy) ? m_new : m_old;
+      m_safe[rt] = (m_use == kNegInf) ? 0.f : m_use;
+      alpha_cur[rt] = fast_exp2(m_old - m_safe[rt]);
+      m_run[rt] = m_use;
+      psum[rt] = 0.f;
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    mfma_slice(1);
+    exp_slice(0);
+    __builtin_amdgcn_sched_barrier(0);
+    mfma_slice(2);
+    exp_slice(8);
+    pack_slice(0);
+    __builtin_amdgcn_sched_barrier(0);
+    mfma_slice(3);
+    pack_slice(1);
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) l_run[rt] = l_run[rt] * alpha_cur[rt] + psum[rt];
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  auto half_step = [&](Scores& cur, int cur_base, bool need_mask, Scores& nxt, int k_buf, int k_kt,
+                       int v_buf, int v_kt, const bf16x8_t (&pb_prev)[RT][2],
+                       const float (&alpha_prev)[RT], bf16x8_t (&pb_cur)[RT][2],
+                       float (&alpha_cur)[RT]) {
+    rescale(alpha_prev);
+    float mul = p.scale_log2e;
+    if (need_mask) {  // boundary halves: scale and mask in place, in a block of their own
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int key = cur_base + 8 * (i >> 2) + 4 * h + (i & 3);
+          const float x = cur.s[rt][i] * p.scale_log2e;
+          cur.s[rt][i] = (key < row_lo[rt] || key > row_hi[rt]) ? kNegInf : x;
+        }
+      mul = 1.0f;
+    }
+    fused_half(cur, mul, nxt, k_buf, k_kt, v_buf, v_kt, pb_prev, pb_cur, alpha_cur);
+  };
 
   // ---- main loop ---------------------------------------------------------------------
-  // Every load and LDS store below is unconditional (tiles past the end clamp to the last
-  // key and are never read), so the loop body has one fixed sequence of memory operations:
-  // the next tile's rows are in flight during the whole compute phase and the slot ids of
-  // the tile after it were fetched a full iteration earlier.
+  // Four LDS stages: tiles j-1 (V of its second half), j, j+1 (K of its first half) and the
+  // stage being filled with tile j+2.  Every load and LDS store is unconditional (tiles past
+  // the end clamp to the last key and are fully masked), so each wait is a compile-time
+  // partial wait.  Rows travel HBM -> registers -> LDS with a full iteration in flight:
+  // requested in the middle of iteration j-1, parked in LDS in the middle of iteration j,
+  // first read in iteration j+1.
+  const bool general_scale = p.scale_log2e <= 0.f;  // fast path needs a positive scale
   if (n_tiles > 0) {
     slot_load(k_lo);
     stage_load();
     slot_load(k_lo + kBN);
     stage_store(0);
+    stage_load();
+    slot_load(k_lo + 2 * kBN);
+    stage_store(1);
+    stage_load();               // rows of tile 2 stay in registers into the first iteration
+    slot_load(k_lo + 3 * kBN);
     __syncthreads();
-    for (int t = 0; t < n_tiles; ++t) {
-      const int tb = k_lo + t * kBN;
-      stage_load();                // rows of tile t+1
-      slot_load(tb + 2 * kBN);     // slot ids of tile t+2
-      if (tb <= w_hi_max && tb + kBN - 1 >= w_lo_min) compute_tile(t & 1, tb);
-      stage_store((t + 1) & 1);
-      __syncthreads();
+    Scores sa, sb;
+    qk_half(0, 0, sa);
+    bf16x8_t pb_a[RT][2], pb_b[RT][2];
+    float alpha_a[RT], alpha_b[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      alpha_b[rt] = 1.0f;
+#pragma unroll
+      for (int u = 0; u < 2; ++u) pb_b[rt][u] = as_bf16x8(u32x4_t{0u, 0u, 0u, 0u});
     }
+    // stage indices of tiles j-1, j, j+1, j+2 (the first P is zero, so "tile -1" may alias 0)
+    int b_prev = 0, b_cur = 0, b_next = 1, b_fill = 2, b_spare = 3;
+#ifdef MSGL_PROFILE_PHASES
+    long long prof_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    long long prof_t = clock64();
+    const long long prof_c0 = prof_t, prof_w0 = wall_clock64();
+#endif
+    for (int j = 0; j < n_tiles; ++j) {
+      const int tb = k_lo + j * kBN;
+      const bool m0 = general_scale || (tb < w_lo_max) || (tb + 31 > w_hi_min);
+      const bool m1 = general_scale || (tb + 32 < w_lo_max) || (tb + 63 > w_hi_min);
+      // half (j,0): scores of (j,1) from K stage j, P V of (j-1,1) from V stage j-1
+      half_step(sa, tb, m0, sb, b_cur, 1, b_prev, 1, pb_b, alpha_b, pb_a, alpha_a);
+      MSGL_TICK(1);
+      // rows of tile j+2 were requested an iteration ago: park them in the free stage, then
+      // request tile j+3 (its slot ids were fetched an iteration ago as well)
+      stage_store(b_fill);
+      MSGL_TICK(3);
+      stage_load();
+      slot_load(tb + 4 * kBN);
+      MSGL_TICK(0);
+      // half (j,1): scores of (j+1,0) from K stage j+1, P V of (j,0) from V stage j
+      half_step(sb, tb + 32, m1, sa, b_next, 0, b_cur, 0, pb_a, alpha_a, pb_b, alpha_b);
+      MSGL_TICK(2);
+      __syncthreads();
+      MSGL_TICK(4);
+      const int freed = (j == 0) ? b_spare : b_prev;  // stage of tile j-1 is free after this barrier
+      b_prev = b_cur;
+      b_cur = b_next;
+      b_next = b_fill;
+      b_fill = freed;
+    }
+    // the last half's P V is still owed
+    rescale(alpha_b);
+    pv_half(b_prev, 1, pb_b);
+    __syncthreads();  // the epilogue reuses the stages as its output staging area
+#ifdef MSGL_PROFILE_PHASES
+    if (lane == 0) {
+      long long* dst = p.prof + ((long long)blockIdx.x * 8 + w) * 8;
+      for (int i = 0; i < 5; ++i) dst[i] = prof_acc[i];
+      dst[5] = n_tiles;
+      dst[6] = clock64() - prof_c0;
+      dst[7] = wall_clock64() - prof_w0;
+    }
+#endif
   }
 
   // ---- epilogue: normalise, un-permute through LDS, store whole rows -----------------
@@ -367,6 +557,10 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
 
 }  // namespace
 
+#ifdef MSGL_PROFILE_PHASES
+static long long* g_prof_buf = nullptr;
+extern "C" __attribute__((visibility("default"))) long long* msgl_debug_prof_buffer() { return g_prof_buf; }
+#endif
 static std::atomic<int> g_tile_variant{0};
 int tile_variant() { return g_tile_variant.load(); }
 void set_tile_variant(int v) { g_tile_variant.store(v); }
@@ -392,6 +586,12 @@ int launch_prefill_tile(const PrefillArgs& a, hipStream_t stream) {
   p.is_cross = a.is_cross;
   p.window = a.window;
   p.scale_log2e = a.sm_scale * kLog2e;
+#ifdef MSGL_PROFILE_PHASES
+  static long long* prof_buf = nullptr;
+  if (!prof_buf) (void)hipMalloc(&prof_buf, 8192 * 64 * sizeof(long long));
+  p.prof = prof_buf;
+  g_prof_buf = prof_buf;
+#endif
   const int variant = tile_variant();
   const int64_t block_rows = 256;
   const int64_t rows = (int64_t)a.max_len_extend * p.group;
@@ -402,12 +602,16 @@ int launch_prefill_tile(const PrefillArgs& a, hipStream_t stream) {
   if (n_blocks > 0x7fffffffLL) return MSGL_ERR_SHAPE;
   p.n_qblk = (int32_t)n_qblk;
   p.n_pairs = (int32_t)n_pairs;
-  if (variant == 1)
-    hipLaunchKernelGGL((prefill_tile_kernel<128, 2, 4>), dim3((unsigned)n_blocks), dim3(256), 0,
-                       stream, p);
-  else
-    hipLaunchKernelGGL((prefill_tile_kernel<128, 1, 8>), dim3((unsigned)n_blocks), dim3(512), 0,
-                       stream, p);
+  const bool wide = (uint64_t)a.num_slots * (uint64_t)a.k_stride0 * 2u >= (1ull << 32) ||
+                    (uint64_t)a.num_slots * (uint64_t)a.v_stride0 * 2u >= (1ull << 32);
+  const dim3 grid((unsigned)n_blocks);
+  if (variant == 1) {
+    if (wide) hipLaunchKernelGGL((prefill_tile_kernel<128, 2, 4, true>), grid, dim3(256), 0, stream, p);
+    else hipLaunchKernelGGL((prefill_tile_kernel<128, 2, 4, false>), grid, dim3(256), 0, stream, p);
+  } else {
+    if (wide) hipLaunchKernelGGL((prefill_tile_kernel<128, 1, 8, true>), grid, dim3(512), 0, stream, p);
+    else hipLaunchKernelGGL((prefill_tile_kernel<128, 1, 8, false>), grid, dim3(512), 0, stream, p);
+  }
   return check_launch();
 }
 
