@@ -204,11 +204,12 @@ def run_config(cfg: int, variant: str, steps: int, warmup: int, check: bool, cpu
 
 
 def load_traffic():
-    """Measured HBM bytes per launch from the committed rocprofv3 counter summaries."""
+    """Measured HBM bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, calibrated against a
+    copy of known size) for the workloads that have a committed counter summary."""
     path = os.path.join(ROOT, "profiles", "hbm_traffic.json")
     if os.path.exists(path):
         with open(path) as f:
-            return json.load(f)
+            return {k: v.get("total_bytes") for k, v in json.load(f).items()}
     return {}
 
 
@@ -222,6 +223,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--tune", action="append", default=[], metavar="KNOB=VALUE",
                     help="set a msgl_set_tuning knob (benchmarking only), e.g. 0=512")
+    ap.add_argument("--copy-probe-mib", type=int, default=0,
+                    help="also run one device-to-device copy of this many MiB (a kernel of "
+                         "known traffic that calibrates rocprofv3 FETCH_SIZE / WRITE_SIZE)")
     ap.add_argument("--cpu-flops", type=float, default=3e11,
                     help="flop budget of the CPU baseline sample per shape")
     args = ap.parse_args()
@@ -242,6 +246,14 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     traffic = load_traffic()
+    if args.copy_probe_mib > 0:
+        n = args.copy_probe_mib << 20
+        src = torch.empty(n, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        dst.copy_(src)  # reads n bytes, writes n bytes
+        torch.cuda.synchronize()
+        log(f"[copy probe] {args.copy_probe_mib} MiB device copy done")
+        del src, dst
 
     rows = []
     for tok in [t.strip() for t in args.configs.split(",") if t.strip()]:
