@@ -148,6 +148,7 @@ int msgl_paged_decode_attention(const void* q, const void* k_cache, const void* 
   a.n_q = num_q_heads;
   a.n_kv = num_kv_heads;
   a.head_dim = head_dim;
+  a.num_slots = num_slots;
   a.k_stride0 = k_cache_stride0;
   a.v_stride0 = v_cache_stride0;
   a.sm_scale = sm_scale;
@@ -220,6 +221,7 @@ int msgl_paged_prefill_attention(const void* q, const void* k_cache, const void*
     a.n_q = num_q_heads;
     a.n_kv = num_kv_heads;
     a.head_dim = head_dim;
+    a.num_slots = num_slots;
     a.k_stride0 = k_cache_stride0;
     a.v_stride0 = v_cache_stride0;
     a.sm_scale = sm_scale;

@@ -27,7 +27,7 @@ struct SplitKvArgs {
   const int32_t* prefix_lens;  // nullptr for decode
   void* out;
   void* workspace;
-  int64_t batch, total_kv, n_q, n_kv, head_dim;
+  int64_t batch, total_kv, n_q, n_kv, head_dim, num_slots;
   int64_t k_stride0, v_stride0;  // elements
   float sm_scale;
   int32_t max_len_extend;  // 1 for decode

@@ -65,6 +65,7 @@ struct SplitKvParams {
   int32_t head_groups;  // n_kv / nwh
   int32_t n_seg, min_seg, cols, max_len_extend;
   int32_t is_cross, window;
+  int32_t wide;  // pool byte offsets need 64 bits
   float scale_log2e;
 };
 
@@ -161,7 +162,9 @@ struct KvTile {
 
 // NCT = tiles of 16 columns per wave, NW = waves per workgroup (launch bound only).  One
 // column tile at head dim 128 fits 256 VGPRs, so two such waves per SIMD can be resident.
-template <int D, int NCT, int NW>
+// WIDE: pool byte offsets need 64 bits (a pool of 4 GiB or more); otherwise a row's offset is
+// one 32-bit multiply instead of a 64-bit multiply-add per load.
+template <int D, int NCT, int NW, bool WIDE>
 __global__ __launch_bounds__(64 * NW, ((D == 128 && NCT == 1) ? 2 : 1)) void splitkv_attention_kernel(SplitKvParams p) {
   constexpr int KS = D / 32;   // k-steps of the QK product
   constexpr int VH = D / 128;  // 128-wide halves of D in the PV product
@@ -182,8 +185,16 @@ __global__ __launch_bounds__(64 * NW, ((D == 128 && NCT == 1) ? 2 : 1)) void spl
   int vpos = seg * seg_len;
   const int seg_end = min(vpos + seg_len, total);
 
-  const uint16_t* kbase = p.k_cache + (int64_t)kvh * D + g * 8;
-  const uint16_t* vbase = p.v_cache + (int64_t)kvh * D + t16 * 8;
+  const unsigned char* kbase =
+      reinterpret_cast<const unsigned char*>(p.k_cache + (int64_t)kvh * D + g * 8);
+  const unsigned char* vbase =
+      reinterpret_cast<const unsigned char*>(p.v_cache + (int64_t)kvh * D + t16 * 8);
+  const uint32_t k_row_bytes = (uint32_t)p.k_stride0 * 2u;
+  const uint32_t v_row_bytes = (uint32_t)p.v_stride0 * 2u;
+  auto row_offset = [](int slot_id, uint32_t row_bytes) -> uint64_t {
+    if constexpr (WIDE) return (uint64_t)(uint32_t)slot_id * row_bytes;
+    else return (uint64_t)((uint32_t)slot_id * row_bytes);
+  };
 
   while (vpos < seg_end) {
     const ReqInfo r = request_info(p, cur_b);
@@ -262,8 +273,8 @@ __global__ __launch_bounds__(64 * NW, ((D == 128 && NCT == 1) ? 2 : 1)) void spl
     auto load_tile = [&](KvTile<D>& t, int s0, int s1) {
 #pragma unroll
       for (int c = 0; c < KS; ++c) {
-        t.k[0][c] = ld_global_b128(kbase + (int64_t)s0 * p.k_stride0 + c * 32);
-        t.k[1][c] = ld_global_b128(kbase + (int64_t)s1 * p.k_stride0 + c * 32);
+        t.k[0][c] = ld_global_b128(kbase + row_offset(s0, k_row_bytes) + c * 64);
+        t.k[1][c] = ld_global_b128(kbase + row_offset(s1, k_row_bytes) + c * 64);
       }
       // V rows of this lane group: tokens 4g+j (j<4) of sub-tile 0, then of sub-tile 1;
       // their slot ids sit in lanes 4g+j of the K index registers.
@@ -271,9 +282,9 @@ __global__ __launch_bounds__(64 * NW, ((D == 128 && NCT == 1) ? 2 : 1)) void spl
       for (int j = 0; j < 8; ++j) {
         const int src = 4 * g + (j & 3);
         const int slot = __shfl(j < 4 ? s0 : s1, src, kWave);
-        const uint16_t* vrow = vbase + (int64_t)slot * p.v_stride0;
+        const unsigned char* vrow = vbase + row_offset(slot, v_row_bytes);
 #pragma unroll
-        for (int hf = 0; hf < VH; ++hf) t.v[hf][j] = ld_global_b128(vrow + hf * 128);
+        for (int hf = 0; hf < VH; ++hf) t.v[hf][j] = ld_global_b128(vrow + hf * 256);
       }
     };
 
@@ -526,8 +537,9 @@ int device_cus() {
 
 template <int D, int NCT, int NW>
 void launch_attn(const SplitKvParams& p, hipStream_t stream) {
-  hipLaunchKernelGGL((splitkv_attention_kernel<D, NCT, NW>),
-                     dim3((unsigned)(p.n_seg * p.head_groups)), dim3(64 * NW), 0, stream, p);
+  const dim3 grid((unsigned)(p.n_seg * p.head_groups)), block(64 * NW);
+  if (p.wide) hipLaunchKernelGGL((splitkv_attention_kernel<D, NCT, NW, true>), grid, block, 0, stream, p);
+  else hipLaunchKernelGGL((splitkv_attention_kernel<D, NCT, NW, false>), grid, block, 0, stream, p);
 }
 
 template <int D, int NCT>
@@ -645,6 +657,8 @@ int launch_splitkv(const SplitKvArgs& a, hipStream_t stream) {
   p.is_cross = a.is_cross;
   p.window = a.window;
   p.scale_log2e = a.sm_scale * kLog2e;
+  p.wide = ((uint64_t)a.num_slots * (uint64_t)a.k_stride0 * 2u >= (1ull << 32) ||
+            (uint64_t)a.num_slots * (uint64_t)a.v_stride0 * 2u >= (1ull << 32)) ? 1 : 0;
   if ((int64_t)p.n_seg * p.head_groups > 0x7fffffffLL) return MSGL_ERR_SHAPE;
   if (a.head_dim == 128) return launch_d<128>(p, nct, stream);
   if (a.head_dim == 256) return launch_d<256>(p, nct, stream);
