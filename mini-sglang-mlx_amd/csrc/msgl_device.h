@@ -36,6 +36,11 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
   return __builtin_bit_cast(uint32_t, p);
 }
 
+// Optimisation barrier on one register value: it must be computed before this point and
+// is treated as modified after it.
+__device__ __forceinline__ void pin(float& x) { asm volatile("" : "+v"(x)); }
+__device__ __forceinline__ void pin(uint32_t& x) { asm volatile("" : "+v"(x)); }
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 // v_perm_b32: result byte i = byte sel[i] of the 8-byte value {hi:lo} (lo = bytes 0..3).

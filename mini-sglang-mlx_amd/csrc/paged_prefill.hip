@@ -351,30 +351,46 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
         smem + k_buf * S::STAGE_BYTES + (k_kt * 32 + c32) * S::KROW * 2 + h * 16;
     const unsigned char* vs =
         smem + v_buf * S::STAGE_BYTES + S::K_BYTES + c32 * S::VROW * 2 + (32 * v_kt + 8 * h) * 2;
-    auto mfma_slice = [&](int sl) {
+    // MFMA operands of one slice: two K rows-of-16-dims and two V^T rows-of-16-keys per lane
+    struct Ops {
+      bf16x8_t k[2], v[2];
+    };
+    auto load_ops = [&](int sl) {
+      Ops o;
+      const int u = sl >> 1;
+#pragma unroll
+      for (int e = 0; e < 2; ++e) {
+        o.k[e] = as_bf16x8(*reinterpret_cast<const u32x4_t*>(ks + (2 * sl + e) * 32));
+        o.v[e] = as_bf16x8(*reinterpret_cast<const u32x4_t*>(
+            vs + (2 * (sl & 1) + e) * 32 * S::VROW * 2 + u * 32));
+      }
+      return o;
+    };
+    auto mfma_slice = [&](int sl, const Ops& o) {
       // alternate the two products: consecutive score MFMAs extend the same accumulator
       // chain, the P V ones go to different accumulators
       const int u = sl >> 1;
 #pragma unroll
       for (int e = 0; e < 2; ++e) {
         const int kstep = 2 * sl + e;
-        const bf16x8_t a = as_bf16x8(*reinterpret_cast<const u32x4_t*>(ks + kstep * 32));
 #pragma unroll
-        for (int rt = 0; rt < RT; ++rt) nxt.s[rt] = mfma_32x32x16(a, qreg[rt][kstep], nxt.s[rt]);
+        for (int rt = 0; rt < RT; ++rt) nxt.s[rt] = mfma_32x32x16(o.k[e], qreg[rt][kstep], nxt.s[rt]);
         const int dt = 2 * (sl & 1) + e;
-        const bf16x8_t b = as_bf16x8(
-            *reinterpret_cast<const u32x4_t*>(vs + dt * 32 * S::VROW * 2 + u * 32));
 #pragma unroll
-        for (int rt = 0; rt < RT; ++rt) oacc[dt][rt] = mfma_32x32x16(b, pb_prev[rt][u], oacc[dt][rt]);
+        for (int rt = 0; rt < RT; ++rt) oacc[dt][rt] = mfma_32x32x16(o.v[e], pb_prev[rt][u], oacc[dt][rt]);
       }
     };
     float m_safe[RT], psum[RT];
+    // pin(): the value must exist at this point of the instruction stream.  Without it the
+    // optimiser sinks the softmax arithmetic out of its slice, next to its first use in the
+    // following step, and the MFMAs of this step run with the VALU idle.
     auto exp_slice = [&](int first) {  // elements first .. first+7
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
         for (int i = first; i < first + 8; ++i) {
-          const float e = fast_exp2(__builtin_fmaf(cur.s[rt][i], mul, -m_safe[rt]));
+          float e = fast_exp2(__builtin_fmaf(cur.s[rt][i], mul, -m_safe[rt]));
+          pin(e);
           cur.s[rt][i] = e;
           psum[rt] += e;
         }
@@ -384,17 +400,23 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
       for (int rt = 0; rt < RT; ++rt) {
         u32x4_t pk;
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-          pk[j] = pack_bf16x2(cur.s[rt][8 * u + 2 * j], cur.s[rt][8 * u + 2 * j + 1]);
+        for (int j = 0; j < 4; ++j) {
+          uint32_t w = pack_bf16x2(cur.s[rt][8 * u + 2 * j], cur.s[rt][8 * u + 2 * j + 1]);
+          pin(w);
+          pk[j] = w;
+        }
         pb_cur[rt][u] = as_bf16x8(pk);
       }
     };
-    // slice 0: row max, lazy-max decision
+    // slice 0: row max, lazy-max decision.  Each slice first requests the operands of the
+    // next one, so LDS latency is covered by a slice of MFMA + VALU work.
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
       for (int i = 0; i < 16; ++i) nxt.s[rt][i] = 0.f;
-    mfma_slice(0);
+    const Ops o0 = load_ops(0);
+    const Ops o1 = load_ops(1);
+    mfma_slice(0, o0);
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
       float mx = fmaxf(cur.s[rt][0], cur.s[rt][1]);
@@ -408,16 +430,20 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
       alpha_cur[rt] = fast_exp2(m_old - m_safe[rt]);
       m_run[rt] = m_use;
       psum[rt] = 0.f;
+      pin(m_safe[rt]);
+      pin(alpha_cur[rt]);
     }
     __builtin_amdgcn_sched_barrier(0);
-    mfma_slice(1);
+    const Ops o2 = load_ops(2);
+    mfma_slice(1, o1);
     exp_slice(0);
     __builtin_amdgcn_sched_barrier(0);
-    mfma_slice(2);
+    const Ops o3 = load_ops(3);
+    mfma_slice(2, o2);
     exp_slice(8);
     pack_slice(0);
     __builtin_amdgcn_sched_barrier(0);
-    mfma_slice(3);
+    mfma_slice(3, o3);
     pack_slice(1);
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) l_run[rt] = l_run[rt] * alpha_cur[rt] + psum[rt];
