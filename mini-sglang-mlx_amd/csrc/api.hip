@@ -4,6 +4,8 @@
 // and sizes can express them; rank and dtype-equality checks live in the Python shim.
 #include <atomic>
 
+#include <algorithm>
+
 #include "msgl_internal.h"
 
 namespace {
@@ -163,6 +165,14 @@ int msgl_paged_decode_attention(const void* q, const void* k_cache, const void* 
 static bool use_splitkv_route(int64_t group, int64_t max_len_extend) {
   return max_len_extend >= 1 && group * max_len_extend <= smallq_max_cols();
 }
+// The MFMA tile kernel exists for head_dim 128.  Longer queries at head_dim 256 run the
+// split-K kernel once per chunk of queries (each launch re-reads the visible keys).
+static bool use_chunked_route(int64_t head_dim, int64_t group) {
+  return head_dim != 128 && group <= msgl::kSplitKvMaxCols;
+}
+static int32_t chunk_queries(int64_t group) {
+  return (int32_t)std::max<int64_t>(1, std::min<int64_t>(smallq_max_cols(), msgl::kSplitKvMaxCols) / group);
+}
 
 size_t msgl_paged_prefill_workspace_bytes(int64_t batch, int64_t total_q, int64_t total_kv,
                                           int64_t num_q_heads, int64_t num_kv_heads,
@@ -172,7 +182,12 @@ size_t msgl_paged_prefill_workspace_bytes(int64_t batch, int64_t total_q, int64_
       num_q_heads % num_kv_heads != 0)
     return 0;
   const int64_t group = num_q_heads / num_kv_heads;
-  if (!use_splitkv_route(group, max_len_extend)) return 0;
+  if (!use_splitkv_route(group, max_len_extend)) {
+    if (!use_chunked_route(head_dim, group)) return 0;
+    const int32_t qc = chunk_queries(group);
+    return msgl::splitkv_workspace_bytes(batch, num_q_heads, num_kv_heads, head_dim, qc,
+                                         segments(total_kv, num_kv_heads, head_dim, group * qc));
+  }
   return msgl::splitkv_workspace_bytes(
       batch, num_q_heads, num_kv_heads, head_dim, max_len_extend,
       segments(total_kv, num_kv_heads, head_dim, group * max_len_extend));
@@ -201,10 +216,12 @@ int msgl_paged_prefill_attention(const void* q, const void* k_cache, const void*
     return MSGL_ERR_NULL_POINTER;
   const int64_t group = num_q_heads / num_kv_heads;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (use_splitkv_route(group, max_len_extend)) {
-    const int32_t n_seg = segments(total_kv, num_kv_heads, head_dim, group * max_len_extend);
+  const bool direct = use_splitkv_route(group, max_len_extend);
+  if (direct || use_chunked_route(head_dim, group)) {
+    const int32_t per_launch = direct ? max_len_extend : chunk_queries(group);
+    const int32_t n_seg = segments(total_kv, num_kv_heads, head_dim, group * per_launch);
     const size_t need = msgl::splitkv_workspace_bytes(batch, num_q_heads, num_kv_heads, head_dim,
-                                                      max_len_extend, n_seg);
+                                                      per_launch, n_seg);
     if (!workspace || workspace_bytes < need || !aligned16(workspace)) return MSGL_ERR_WORKSPACE;
     msgl::SplitKvArgs a{};
     a.q = q;
@@ -225,12 +242,19 @@ int msgl_paged_prefill_attention(const void* q, const void* k_cache, const void*
     a.k_stride0 = k_cache_stride0;
     a.v_stride0 = v_cache_stride0;
     a.sm_scale = sm_scale;
-    a.max_len_extend = max_len_extend;
+    a.max_len_extend = per_launch;
+    a.q_cap = max_len_extend;
     a.is_cross = is_cross_attention ? 1 : 0;
     a.window = sliding_window_size;
     a.n_seg = n_seg;
     a.min_seg = min_segment();
-    return msgl::launch_splitkv(a, s);
+    // launches share the workspace: they run one after the other on the stream
+    for (int32_t q0 = 0; q0 < max_len_extend; q0 += per_launch) {
+      a.q_begin = q0;
+      rc = msgl::launch_splitkv(a, s);
+      if (rc != MSGL_OK) return rc;
+    }
+    return MSGL_OK;
   }
   msgl::PrefillArgs a{};
   a.q = q;

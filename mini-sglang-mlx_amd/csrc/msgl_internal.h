@@ -30,7 +30,9 @@ struct SplitKvArgs {
   int64_t batch, total_kv, n_q, n_kv, head_dim, num_slots;
   int64_t k_stride0, v_stride0;  // elements
   float sm_scale;
-  int32_t max_len_extend;  // 1 for decode
+  int32_t max_len_extend;  // 1 for decode; queries per request handled by this launch
+  int32_t q_begin;         // first query of every request handled by this launch
+  int32_t q_cap;           // cap on a request's query count (0: max_len_extend)
   int32_t is_cross, window;
   int32_t n_seg;    // segments the visible token stream is cut into
   int32_t min_seg;  // smallest segment length in tokens, multiple of 64

@@ -64,6 +64,7 @@ struct SplitKvParams {
   int32_t nwh;          // kv heads per workgroup
   int32_t head_groups;  // n_kv / nwh
   int32_t n_seg, min_seg, cols, max_len_extend;
+  int32_t q_begin, q_cap;  // first query of every request in this launch; cap on a request's queries
   int32_t is_cross, window;
   int32_t wide;  // pool byte offsets need 64 bits
   float scale_log2e;
@@ -87,9 +88,12 @@ __device__ __forceinline__ ReqInfo request_info(const SplitKvParams& p, int b) {
     r.q_len = 1;
     r.prefix = r.kv_len - 1;
   } else {
-    r.q_start = p.qo_indptr[b];
-    r.q_len = min(p.qo_indptr[b + 1] - r.q_start, p.max_len_extend);
-    r.prefix = p.prefix_lens[b];
+    // this launch covers queries q_begin .. q_begin + max_len_extend - 1 of every request
+    const int q0 = p.qo_indptr[b];
+    const int q_all = min(p.qo_indptr[b + 1] - q0, p.q_cap);
+    r.q_start = q0 + p.q_begin;
+    r.q_len = max(min(q_all - p.q_begin, p.max_len_extend), 0);
+    r.prefix = p.prefix_lens[b] + p.q_begin;
   }
   // first query has the lowest window floor, last query the highest causal limit
   r.lo = (p.window > 0) ? max(0, r.prefix - p.window + 1) : 0;
@@ -654,6 +658,8 @@ int launch_splitkv(const SplitKvArgs& a, hipStream_t stream) {
   p.n_seg = a.n_seg;
   p.min_seg = a.min_seg;
   p.max_len_extend = a.max_len_extend;
+  p.q_begin = a.q_begin;
+  p.q_cap = a.q_cap > 0 ? a.q_cap : a.max_len_extend;
   p.is_cross = a.is_cross;
   p.window = a.window;
   p.scale_log2e = a.sm_scale * kLog2e;

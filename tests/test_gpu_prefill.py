@@ -101,6 +101,24 @@ def test_splitk_route_masks(gpu, q_len, is_cross, window):
     _check(wl, gpu, f"split-K route q_len={q_len} cross={is_cross} W={window}")
 
 
+@pytest.mark.parametrize("is_cross,window", MASKS)
+def test_head_dim_256_short_and_long_queries(gpu, is_cross, window):
+    # head_dim 256 has no MFMA tile kernel: short query blocks take the split-K route in one
+    # launch, longer ones run it once per chunk of queries (here 64 / group = 16 per launch;
+    # extends of 5, 16, 40 and 70 give a request that ends inside the first chunk, one that
+    # fills it exactly, and two that span three and five chunks)
+    wl = build_workload("t", "prefill", seed=330, n_q=8, n_kv=2, head_dim=256,
+                        kv_lens=[5, 100 + 16, 300 + 40, 70], extend_lens=[5, 16, 40, 70],
+                        pool_factor=1.2, store_new=True,
+                        is_cross_attention=is_cross, sliding_window_size=window)
+    _check(wl, gpu, f"head_dim 256 chunked cross={is_cross} W={window}")
+    short = build_workload("t", "prefill", seed=331, n_q=8, n_kv=2, head_dim=256,
+                           kv_lens=[7, 200 + 7, 64 + 3], extend_lens=[7, 7, 3], pool_factor=1.2,
+                           store_new=True, is_cross_attention=is_cross,
+                           sliding_window_size=window)
+    _check(short, gpu, f"head_dim 256 short cross={is_cross} W={window}")
+
+
 def test_splitk_route_ragged_q_and_chunking(gpu):
     from mini_sglang_amd_kernel import _lib
 
