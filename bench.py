@@ -213,6 +213,33 @@ def load_traffic():
     return {}
 
 
+def mfma_rate_probe():
+    """Sustained v_mfma_f32_32x32x16_bf16 rate of the whole chip on register-resident operands,
+    nothing else running: all-zero operands and N(0,1) operands that change every instruction.
+    The board lowers its shader clock to hold its power limit and MFMA power grows with the
+    number of toggling operand bits, so the second figure, not the datasheet peak, is what a
+    kernel on random bf16 data can reach."""
+    import ctypes
+
+    path = os.path.join(ROOT, "mini-sglang-mlx_amd", "lib", "libmsgl_probes.so")
+    if not os.path.exists(path):
+        return None
+    lib = ctypes.CDLL(path)
+    lib.msgl_probe_mfma_rate.restype = ctypes.c_int
+    lib.msgl_probe_mfma_rate.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_double),
+                                         ctypes.POINTER(ctypes.c_double)]
+    out = {"unit": "TFLOP/s", "kernel": "back-to-back v_mfma_f32_32x32x16_bf16, 4 waves per CU"}
+    for name, mode in (("zero_operands", 0), ("random_operands", 1)):
+        tf, ghz = ctypes.c_double(0), ctypes.c_double(0)
+        rc = lib.msgl_probe_mfma_rate(mode, 40000, ctypes.byref(tf), ctypes.byref(ghz))
+        if rc != 0:
+            return None
+        out[name] = tf.value
+        out[name + "_shader_ghz"] = ghz.value
+        log(f"[mfma probe] {name}: {tf.value:.0f} TFLOP/s at {ghz.value:.2f} GHz")
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -226,6 +253,10 @@ def main():
     ap.add_argument("--copy-probe-mib", type=int, default=0,
                     help="also run one device-to-device copy of this many MiB (a kernel of "
                          "known traffic that calibrates rocprofv3 FETCH_SIZE / WRITE_SIZE)")
+    ap.add_argument("--no-mfma-probe", action="store_true",
+                    help="skip the measurement of the matrix pipe's sustained rate on zero and "
+                         "on random operands (the power-limited ceiling the prefill figure is "
+                         "reported beside)")
     ap.add_argument("--cpu-flops", type=float, default=3e11,
                     help="flop budget of the CPU baseline sample per shape")
     args = ap.parse_args()
@@ -319,6 +350,8 @@ def main():
             "roofline": roofline_obj(pre), "cpu_baseline": cpu_obj(pre),
             "parity_ok": pre.get("parity_ok"), "kv_pool_bit_exact": pre.get("kv_pool_bit_exact"),
         }
+        if not args.no_mfma_probe:
+            result["prefill"]["mfma_rate_probe"] = mfma_rate_probe()
     result["all_configs"] = rows
     print(json.dumps(result))
 

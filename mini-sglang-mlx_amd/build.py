@@ -17,6 +17,9 @@ CSRC = os.path.join(HERE, "csrc")
 LIB_DIR = os.path.join(HERE, "lib")
 OBJ_DIR = os.path.join(HERE, "build")
 LIB_PATH = os.path.join(LIB_DIR, "libmsgl_paged_attention.so")
+# benchmarking aid (measured MFMA ceiling under the board's power limit); bench.py loads it
+PROBE_SRC = os.path.join(CSRC, "probes", "mfma_rate_probe.hip")
+PROBE_PATH = os.path.join(LIB_DIR, "libmsgl_probes.so")
 SOURCES = ["api.hip", "store_kv_cache.hip", "paged_splitkv.hip", "paged_prefill.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
@@ -68,6 +71,11 @@ def build(force: bool = False, save_temps: bool = False) -> str:
         proc = subprocess.run(cmd, capture_output=True, text=True)
         if proc.returncode != 0:
             raise RuntimeError(f"link failed:\n{proc.stderr}")
+    if force or _newer([PROBE_SRC], PROBE_PATH):
+        cmd = [HIPCC, *FLAGS, "-shared", PROBE_SRC, "-o", PROBE_PATH]
+        proc = subprocess.run(cmd, capture_output=True, text=True)
+        if proc.returncode != 0:
+            raise RuntimeError(f"hipcc failed for the probe library:\n{proc.stderr}")
     return LIB_PATH
 
 

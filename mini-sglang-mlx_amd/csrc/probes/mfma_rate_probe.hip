@@ -1,0 +1,107 @@
+// What the matrix pipe sustains on this board when nothing else runs: back-to-back
+// v_mfma_f32_32x32x16_bf16 on register-resident operands, one workgroup of four waves per CU.
+// The board holds a power limit by lowering the shader clock, and MFMA power depends on how
+// many operand bits toggle, so the rate is measured for all-zero operands and for operands
+// drawn from N(0,1) that change with every instruction.  The second figure is the ceiling a
+// bf16 attention kernel on random data is measured against; the datasheet peak assumes the
+// boost clock.  Benchmarking aid only: not part of the paged-attention library.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace {
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+
+__device__ uint32_t mix(uint32_t x) {
+  x ^= x >> 16;
+  x *= 0x7feb352dU;
+  x ^= x >> 15;
+  x *= 0x846ca68bU;
+  x ^= x >> 16;
+  return x;
+}
+// roughly N(0,1): centred sum of four uniforms
+__device__ float draw(uint32_t seed) {
+  float s = 0.f;
+  for (int i = 0; i < 4; ++i) {
+    seed = mix(seed + i * 0x9e3779b9U);
+    s += (seed >> 8) * (1.0f / 16777216.0f);
+  }
+  return (s - 2.0f) * 1.7320508f;
+}
+
+__global__ __launch_bounds__(256) void mfma_rate_kernel(int random_operands, int iters, float* sink,
+                                                        long long* clocks) {
+  f32x16_t acc[4];
+  for (int a = 0; a < 4; ++a)
+    for (int i = 0; i < 16; ++i) acc[a][i] = 0.f;
+  bf16x8_t av[8], bv[8];
+  const uint32_t tid = blockIdx.x * 256 + threadIdx.x;
+  for (int r = 0; r < 8; ++r)
+    for (int i = 0; i < 8; ++i) {
+      av[r][i] = (__bf16)(random_operands ? draw(tid * 131 + r * 17 + i) : 0.f);
+      bv[r][i] = (__bf16)(random_operands ? draw(tid * 257 + r * 29 + i + 1000) : 0.f);
+    }
+  const long long c0 = clock64(), w0 = wall_clock64();
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int r = 0; r < 8; ++r)
+      acc[r & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[r], bv[r], acc[r & 3], 0, 0, 0);
+    if ((it & 255) == 255)  // keep the sums finite
+      for (int a = 0; a < 4; ++a)
+        for (int i = 0; i < 16; ++i) acc[a][i] *= 1e-3f;
+  }
+  const long long c1 = clock64(), w1 = wall_clock64();
+  float s = 0.f;
+  for (int a = 0; a < 4; ++a)
+    for (int i = 0; i < 16; ++i) s += acc[a][i];
+  sink[tid] = s;
+  if (threadIdx.x == 0) {
+    clocks[blockIdx.x * 2] = c1 - c0;
+    clocks[blockIdx.x * 2 + 1] = w1 - w0;
+  }
+}
+
+}  // namespace
+
+// Runs the probe on the current device (blocking).  tflops: achieved MFMA rate; shader_ghz:
+// shader clock during the run (cycle counter against the 100 MHz wall counter).
+// Returns 0, or a hipError_t value.
+extern "C" __attribute__((visibility("default"))) int msgl_probe_mfma_rate(int random_operands,
+                                                                         int iters, double* tflops,
+                                                                         double* shader_ghz) {
+  int dev = 0, cus = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+  if (e != hipSuccess) return (int)e;
+  float* sink = nullptr;
+  long long* clocks = nullptr;
+  e = hipMalloc(&sink, (size_t)cus * 256 * sizeof(float));
+  if (e != hipSuccess) return (int)e;
+  e = hipMalloc(&clocks, (size_t)cus * 2 * sizeof(long long));
+  if (e != hipSuccess) {
+    (void)hipFree(sink);
+    return (int)e;
+  }
+  hipEvent_t t0, t1;
+  (void)hipEventCreate(&t0);
+  (void)hipEventCreate(&t1);
+  hipLaunchKernelGGL(mfma_rate_kernel, dim3(cus), dim3(256), 0, 0, random_operands, iters / 10 + 1, sink, clocks);
+  (void)hipEventRecord(t0, 0);
+  hipLaunchKernelGGL(mfma_rate_kernel, dim3(cus), dim3(256), 0, 0, random_operands, iters, sink, clocks);
+  (void)hipEventRecord(t1, 0);
+  e = hipEventSynchronize(t1);
+  float ms = 0.f;
+  (void)hipEventElapsedTime(&ms, t0, t1);
+  long long c[2] = {0, 1};
+  (void)hipMemcpy(c, clocks, sizeof(c), hipMemcpyDeviceToHost);
+  *tflops = (double)cus * 4.0 * iters * 8.0 * 32768.0 / (ms * 1e-3) / 1e12;
+  *shader_ghz = (double)c[0] / (double)c[1] * 0.1;
+  (void)hipEventDestroy(t0);
+  (void)hipEventDestroy(t1);
+  (void)hipFree(sink);
+  (void)hipFree(clocks);
+  return (int)e;
+}

@@ -33,6 +33,9 @@ def test_library_loads_and_exports_every_declared_symbol():
     assert _lib.strerror(0) == "ok"
     assert "head_dim" in _lib.strerror(-2)
     assert _lib.strerror(-9999) == "unknown error code"
+    # the benchmarking aid bench.py loads next to it
+    probes = ctypes.CDLL(os.path.join(os.path.dirname(_lib.LIB_PATH), "libmsgl_probes.so"))
+    assert hasattr(probes, "msgl_probe_mfma_rate")
 
 
 def test_c_abi_argument_checks_return_codes_without_touching_a_gpu():
