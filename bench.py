@@ -213,6 +213,52 @@ def load_traffic():
     return {}
 
 
+def run_metadata_build(dev, steps: int, warmup: int, cpu_baseline: bool):
+    """On-device build of a step's CSR metadata from the slot table, at the sizes of shape 2
+    (64 requests, ~295 K kv tokens) and shape 4 (16 requests, ~1.3 M kv tokens).  Integer copy
+    work: 8 bytes per kv token (slot id read + written) plus 4 per request array entry."""
+    import numpy as np
+    import torch
+
+    from mini_sglang_amd_kernel import build_attention_metadata
+
+    rows_out = []
+    for name, batch, lo, hi in (("shape2_sizes", 64, 1024, 8192), ("shape4_sizes", 16, 32768, 131072)):
+        g = torch.Generator().manual_seed(0x5EED0100 + batch)
+        kv = torch.randint(lo, hi + 1, (batch,), generator=g, dtype=torch.int32)
+        table = torch.randint(0, 2 ** 31 - 1, (batch + 1, hi), generator=g, dtype=torch.int32)
+        trows = torch.randperm(batch, generator=g).to(torch.int32)
+        total = int(kv.sum())
+        d_table, d_rows, d_kv = table.to(dev), trows.to(dev), kv.to(dev)
+
+        def step():
+            return build_attention_metadata(d_table, d_rows, d_kv, None, total_kv=total)
+
+        out = step()
+        torch.cuda.synchronize()
+        mean_ms, per, _ = time_steps(step, steps, warmup)
+        abytes = 8 * total + 4 * (5 * batch + 2)
+        row = {"sizes": name, "batch": batch, "total_kv_tokens": total, "us_mean": mean_ms * 1e3,
+               "us_min": min(per) * 1e3, "algorithmic_bytes": abytes,
+               "achieved_GBps": abytes / (mean_ms * 1e-3) / 1e9}
+        if cpu_baseline:
+            from oracle import metadata_oracle  # checker and CPU baseline only
+
+            t1 = time.perf_counter()
+            want = metadata_oracle.build_decode_metadata(table.numpy(), trows.numpy(), kv.numpy())
+            cpu_s = time.perf_counter() - t1
+            row["cpu_port_us"] = cpu_s * 1e6
+            row["exact"] = bool(np.array_equal(out["kv_indices"].cpu().numpy(), want["kv_indices"])
+                                and np.array_equal(out["kv_indptr"].cpu().numpy(), want["kv_indptr"])
+                                and np.array_equal(out["num_kv_splits"].cpu().numpy(),
+                                                   want["num_kv_splits"]))
+        log(f"[metadata] {name}: {row['us_mean']:.1f} us mean ({row['us_min']:.1f} min)  "
+            f"{row['achieved_GBps']:.0f} GB/s  cpu {row.get('cpu_port_us', float('nan')):.0f} us  "
+            f"exact {row.get('exact')}")
+        rows_out.append(row)
+    return rows_out
+
+
 def mfma_rate_probe():
     """Sustained v_mfma_f32_32x32x16_bf16 rate of the whole chip on register-resident operands,
     nothing else running: all-zero operands and N(0,1) operands that change every instruction.
@@ -253,6 +299,8 @@ def main():
     ap.add_argument("--copy-probe-mib", type=int, default=0,
                     help="also run one device-to-device copy of this many MiB (a kernel of "
                          "known traffic that calibrates rocprofv3 FETCH_SIZE / WRITE_SIZE)")
+    ap.add_argument("--no-metadata", action="store_true",
+                    help="skip the on-device metadata build (slot table -> CSR arrays) figures")
     ap.add_argument("--no-mfma-probe", action="store_true",
                     help="skip the measurement of the matrix pipe's sustained rate on zero and "
                          "on random operands (the power-limited ceiling the prefill figure is "
@@ -352,6 +400,9 @@ def main():
         }
         if not args.no_mfma_probe:
             result["prefill"]["mfma_rate_probe"] = mfma_rate_probe()
+    if not args.no_metadata:
+        result["metadata_build"] = run_metadata_build(dev, args.steps, args.warmup,
+                                                      not args.no_cpu_baseline)
     result["all_configs"] = rows
     print(json.dumps(result))
 

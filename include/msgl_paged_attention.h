@@ -8,6 +8,9 @@
  *   paged_decode_attention    GQA split-K decode over slots gathered through kv_indices
  *   paged_prefill_attention   extend attention (causal / full / window / bidirectional+window)
  *
+ * and the step's metadata build that feeds them (slot table -> CSR arrays), which the
+ * reference does in Python (mini_sglang_mlx/attention/backend.py:205-307).
+ *
  * Conventions shared by every entry point
  *   - every pointer is a DEVICE pointer in the address space of the current HIP
  *     device; `stream` is a hipStream_t passed as void* (NULL = the null stream);
@@ -145,6 +148,34 @@ MSGL_API int msgl_paged_prefill_attention(const void* q, const void* k_cache, co
                                  int32_t dtype, void* stream);
 
 /*
+ * build_attention_metadata -- replaces AttnBackend.build_prefill_metadata /
+ * build_decode_metadata, _build_indptr and _compute_num_kv_splits
+ * (mini_sglang_mlx/attention/backend.py:205-307) with one launch and no host round trip:
+ *     kv_indptr  = cumsum([0] + kv_lens)          qo_indptr = cumsum([0] + extend_lens)
+ *     kv_indices = concat(page_table[table_rows[b], :kv_lens[b]])
+ *     prefix_lens[b] = kv_lens[b] - extend_lens[b]
+ *     positions  = concat(arange(prefix_lens[b], kv_lens[b]))
+ *     num_kv_splits[b] = min(max_kv_splits, max(1, ceil(kv_lens[b] / 128)))
+ * page_table is the (n_table_rows, max_seq_len) int32 slot table (one slot id per token,
+ * engine.py:84-87) with leading stride `table_stride0` elements; table_rows, kv_lens and
+ * extend_lens are int32 [batch].  extend_lens == NULL means one query per request (decode:
+ * positions[b] = kv_lens[b] - 1, qo_indptr = 0..batch).  qo_indptr, prefix_lens, positions and
+ * num_kv_splits may be NULL (not produced).  Lengths are clamped to [0, max_seq_len]
+ * (extend_lens to [0, kv_len]) and table rows to the table, so no access leaves the
+ * arguments; writes to kv_indices / positions stop at kv_capacity / q_capacity elements while
+ * kv_indptr[batch] / qo_indptr[batch] always hold the full totals, so the caller can detect
+ * a capacity that was too small.  batch <= 8000.
+ */
+MSGL_API int msgl_build_attention_metadata(const int32_t* page_table, int64_t table_stride0,
+                                  int64_t n_table_rows, int64_t max_seq_len,
+                                  const int32_t* table_rows, const int32_t* kv_lens,
+                                  const int32_t* extend_lens, int64_t batch,
+                                  int32_t* kv_indptr, int32_t* kv_indices, int64_t kv_capacity,
+                                  int32_t* qo_indptr, int32_t* prefix_lens, int32_t* positions,
+                                  int64_t q_capacity, int32_t* num_kv_splits,
+                                  int32_t max_kv_splits, void* stream);
+
+/*
  * Tuning knobs, for benchmarking only (0 = built-in heuristic).  Process-wide,
  * read at launch time; not part of the reference surface.
  *   MSGL_TUNE_SEGMENTS       segments the split-K kernel cuts the visible token stream into
@@ -152,6 +183,7 @@ MSGL_API int msgl_paged_prefill_attention(const void* q, const void* k_cache, co
  *   MSGL_TUNE_SMALLQ_MAXCOLS largest q_len*group routed to the split-K kernel
  *   MSGL_TUNE_PREFILL_VARIANT tiling of the MFMA kernel (0: 8 waves x 32 rows, 1: 4 x 64)
  *   MSGL_TUNE_SPLITKV_WAVES  most waves (adjacent kv heads) per split-K workgroup: 1, 2, 4, 8
+ *                            (0 restores the default, 4)
  */
 #define MSGL_TUNE_SEGMENTS 0
 #define MSGL_TUNE_MIN_SEGMENT 1

@@ -281,4 +281,40 @@ int msgl_paged_prefill_attention(const void* q, const void* k_cache, const void*
   return msgl::launch_prefill_tile(a, s);
 }
 
+int msgl_build_attention_metadata(const int32_t* page_table, int64_t table_stride0,
+                                  int64_t n_table_rows, int64_t max_seq_len,
+                                  const int32_t* table_rows, const int32_t* kv_lens,
+                                  const int32_t* extend_lens, int64_t batch, int32_t* kv_indptr,
+                                  int32_t* kv_indices, int64_t kv_capacity, int32_t* qo_indptr,
+                                  int32_t* prefix_lens, int32_t* positions, int64_t q_capacity,
+                                  int32_t* num_kv_splits, int32_t max_kv_splits, void* stream) {
+  if (batch < 0 || batch > msgl::kMetadataMaxBatch || n_table_rows <= 0 || max_seq_len < 0 ||
+      table_stride0 < max_seq_len || kv_capacity < 0 || q_capacity < 0 ||
+      kv_capacity > 0x7fffffffLL || q_capacity > 0x7fffffffLL || max_seq_len > 0x7fffffffLL ||
+      n_table_rows > 0x7fffffffLL)
+    return MSGL_ERR_SHAPE;
+  if (!kv_indptr) return MSGL_ERR_NULL_POINTER;
+  if (batch > 0 && (!page_table || !table_rows || !kv_lens)) return MSGL_ERR_NULL_POINTER;
+  if (kv_capacity > 0 && !kv_indices) return MSGL_ERR_NULL_POINTER;
+  msgl::MetadataArgs a{};
+  a.page_table = page_table;
+  a.table_rows = table_rows;
+  a.kv_lens = kv_lens;
+  a.extend_lens = extend_lens;
+  a.kv_indptr = kv_indptr;
+  a.kv_indices = kv_indices;
+  a.qo_indptr = qo_indptr;
+  a.prefix_lens = prefix_lens;
+  a.positions = positions;
+  a.num_kv_splits = num_kv_splits;
+  a.table_stride0 = table_stride0;
+  a.batch = batch;
+  a.n_table_rows = n_table_rows;
+  a.max_seq_len = max_seq_len;
+  a.kv_capacity = kv_capacity;
+  a.q_capacity = positions ? q_capacity : 0;
+  a.max_kv_splits = max_kv_splits;
+  return msgl::launch_build_metadata(a, static_cast<hipStream_t>(stream));
+}
+
 }  // extern "C"

@@ -1,6 +1,7 @@
 // Host-side declarations shared by the translation units of libmsgl_paged_attention.so.
 #pragma once
 #include <hip/hip_runtime.h>
+#include <algorithm>
 #include <stddef.h>
 #include <stdint.h>
 
@@ -70,6 +71,25 @@ int launch_prefill_tile(const PrefillArgs& a, hipStream_t stream);
 // 1: 4 waves x 64 rows); both cover 256 rows per workgroup
 int tile_variant();
 void set_tile_variant(int v);
+
+// ---- build_metadata.hip ------------------------------------------------------------
+struct MetadataArgs {
+  const int32_t* page_table;
+  const int32_t* table_rows;
+  const int32_t* kv_lens;
+  const int32_t* extend_lens;  // nullptr: decode
+  int32_t* kv_indptr;
+  int32_t* kv_indices;
+  int32_t* qo_indptr;
+  int32_t* prefix_lens;
+  int32_t* positions;
+  int32_t* num_kv_splits;
+  int64_t table_stride0, batch, n_table_rows, max_seq_len, kv_capacity, q_capacity;
+  int32_t max_kv_splits;
+};
+// largest batch one launch handles (two scanned offset arrays live in LDS)
+constexpr int64_t kMetadataMaxBatch = 8000;
+int launch_build_metadata(const MetadataArgs& a, hipStream_t stream);
 
 inline int check_launch() { return hipGetLastError() == hipSuccess ? MSGL_OK : MSGL_ERR_LAUNCH; }
 

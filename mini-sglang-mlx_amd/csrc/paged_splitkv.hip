@@ -583,7 +583,7 @@ int launch_d(const SplitKvParams& p, int nct, hipStream_t stream) {
 
 }  // namespace
 
-void splitkv_set_max_waves(int v) { g_max_waves.store(v); }
+void splitkv_set_max_waves(int v) { g_max_waves.store(v > 0 ? v : 4); }  // 0 restores the default
 
 // kv heads per workgroup for this shape: up to 4, halved when a second wave per head is
 // needed for the columns (a workgroup of the wide variants holds at most 4 waves: they

@@ -15,7 +15,8 @@ from typing import List, Optional, Sequence
 
 import torch
 
-from mini_sglang_amd_kernel import paged_decode_attention, paged_prefill_attention
+from mini_sglang_amd_kernel import (build_attention_metadata, paged_decode_attention,
+                                    paged_prefill_attention)
 
 MAX_KV_SPLITS = 32
 
@@ -117,6 +118,21 @@ class AttnBackend:
         return torch.cat([self.page_table[reqs[i].table_idx, : kv_lens[i]]
                           for i in range(len(reqs))]).to(torch.int32)
 
+    def _device_metadata(self, reqs, kv_lens: Sequence[int],
+                         extend_lens: Optional[Sequence[int]]) -> dict:
+        """One upload of the per-request integers, one kernel for every array (slot table on
+        the GPU).  The host lists are the reference's own inputs (backend.py:228-238)."""
+        device = self.page_table.device
+        host = [[req.table_idx for req in reqs], list(kv_lens)]
+        if extend_lens is not None:
+            host.append(list(extend_lens))
+        packed = torch.tensor(host, dtype=torch.int32).to(device, non_blocking=True)
+        return build_attention_metadata(
+            self.page_table, packed[0], packed[1], packed[2] if extend_lens is not None else None,
+            total_kv=int(sum(kv_lens)),
+            total_q=int(sum(extend_lens)) if extend_lens is not None else len(reqs),
+            max_kv_splits=MAX_KV_SPLITS)
+
     def build_prefill_metadata(self, reqs: List, *, extend_lens: Optional[List[int]] = None,
                                kv_lens: Optional[List[int]] = None,
                                positions: Optional[torch.Tensor] = None) -> PrefillMetadata:
@@ -125,6 +141,13 @@ class AttnBackend:
             extend_lens = [req.extend_len for req in reqs]
         if kv_lens is None:
             kv_lens = [req.device_len for req in reqs]
+        if device.type == "cuda":
+            m = self._device_metadata(reqs, kv_lens, extend_lens)
+            return PrefillMetadata(
+                positions=m["positions"] if positions is None else positions,
+                qo_indptr=m["qo_indptr"], kv_indptr=m["kv_indptr"], kv_indices=m["kv_indices"],
+                prefix_lens=m["prefix_lens"], max_len_extend=max(extend_lens))
+        # slot table in host memory (host-side tests): the same arrays with torch ops
         cached_lens = [kv_lens[i] - extend_lens[i] for i in range(len(reqs))]
         if positions is None:
             positions = torch.cat([
@@ -148,6 +171,11 @@ class AttnBackend:
         if positions is None:
             positions = torch.tensor([req.cached_len for req in reqs], dtype=torch.int32,
                                      device=device)
+        if device.type == "cuda":
+            m = self._device_metadata(reqs, kv_lens, None)
+            return DecodeMetadata(positions=positions, kv_indptr=m["kv_indptr"],
+                                  kv_indices=m["kv_indices"], num_kv_splits=m["num_kv_splits"],
+                                  max_kv_splits=MAX_KV_SPLITS)
         return DecodeMetadata(
             positions=positions,
             kv_indptr=_build_indptr(kv_lens, device),

@@ -20,7 +20,8 @@ import torch
 
 from . import _lib
 
-__all__ = ["store_kv_cache", "paged_decode_attention", "paged_prefill_attention"]
+__all__ = ["store_kv_cache", "paged_decode_attention", "paged_prefill_attention",
+           "build_attention_metadata"]
 
 _DTYPE_CODE = {torch.bfloat16: _lib.MSGL_DTYPE_BF16, torch.float16: _lib.MSGL_DTYPE_F16}
 
@@ -258,5 +259,65 @@ def paged_prefill_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
             _pool_stride0(op, k_cache, "k_cache"), _pool_stride0(op, v_cache, "v_cache"),
             float(sm_scale), int(max_len_extend), int(bool(is_cross_attention)),
             int(sliding_window_size), dtype, _stream_ptr(stream, dev))
+    _check_rc(op, rc)
+    return out
+
+
+def build_attention_metadata(page_table: torch.Tensor, table_rows: torch.Tensor,
+                             kv_lens: torch.Tensor, extend_lens: Optional[torch.Tensor] = None, *,
+                             total_kv: int, total_q: Optional[int] = None,
+                             max_kv_splits: int = 32, stream=None) -> dict:
+    """CSR metadata of one step from the slot table, in one launch on the device.
+
+    Device counterpart of ``AttnBackend.build_prefill_metadata`` / ``build_decode_metadata``
+    (mini_sglang_mlx/attention/backend.py:205-307), which slice the table per request in
+    Python.  ``page_table`` is the ``(rows, max_seq_len)`` int32 slot table, ``table_rows`` /
+    ``kv_lens`` / ``extend_lens`` are int32 ``[batch]`` device tensors; ``extend_lens=None``
+    builds decode metadata (one query per request).  ``total_kv`` / ``total_q`` are the sums
+    of the lengths, which the scheduler knows on the host; they size the outputs.  Returns a
+    dict with ``kv_indptr``, ``kv_indices``, ``qo_indptr``, ``prefix_lens``, ``positions``,
+    ``num_kv_splits``.
+    """
+    op = "build_attention_metadata"
+    if page_table.dim() != 2:
+        _fail(op, "page_table must be 2D (rows, max_seq_len)")
+    if page_table.dtype != torch.int32:
+        _fail(op, "page_table must be int32")
+    if page_table.stride(1) != 1:
+        _fail(op, "page_table must be contiguous in its last dimension")
+    tensors = [page_table, table_rows, kv_lens] + ([extend_lens] if extend_lens is not None else [])
+    for t, name in zip(tensors[1:], ("table_rows", "kv_lens", "extend_lens")):
+        if t.dim() != 1:
+            _fail(op, f"{name} must be 1D")
+    dev = _require_device(op, *tensors)
+    table_rows = _int32_1d(op, table_rows, "table_rows")
+    kv_lens = _int32_1d(op, kv_lens, "kv_lens")
+    batch = kv_lens.shape[0]
+    if table_rows.shape[0] != batch:
+        _fail(op, "table_rows and kv_lens must have the same length")
+    if extend_lens is not None:
+        extend_lens = _int32_1d(op, extend_lens, "extend_lens")
+        if extend_lens.shape[0] != batch:
+            _fail(op, "extend_lens and kv_lens must have the same length")
+    if total_q is None:
+        total_q = batch if extend_lens is None else 0
+    if total_kv < 0 or total_q < 0:
+        _fail(op, "total_kv and total_q must be >= 0")
+    # one allocation, six views (an allocation per array costs more host time than the kernel)
+    sizes = (("kv_indptr", batch + 1), ("qo_indptr", batch + 1), ("prefix_lens", batch),
+             ("num_kv_splits", batch), ("positions", total_q), ("kv_indices", total_kv))
+    buf = torch.empty(sum(n for _, n in sizes), dtype=torch.int32, device=dev)
+    out, at = {}, 0
+    for name, n in sizes:
+        out[name] = buf[at:at + n]
+        at += n
+    rows = page_table.shape[0]
+    stride0 = page_table.stride(0) if rows > 1 else page_table.shape[1]
+    rc = _lib.load().msgl_build_attention_metadata(
+        page_table.data_ptr(), stride0, rows, page_table.shape[1], table_rows.data_ptr(),
+        kv_lens.data_ptr(), extend_lens.data_ptr() if extend_lens is not None else None, batch,
+        out["kv_indptr"].data_ptr(), out["kv_indices"].data_ptr(), total_kv,
+        out["qo_indptr"].data_ptr(), out["prefix_lens"].data_ptr(), out["positions"].data_ptr(),
+        total_q, out["num_kv_splits"].data_ptr(), int(max_kv_splits), _stream_ptr(stream, dev))
     _check_rc(op, rc)
     return out

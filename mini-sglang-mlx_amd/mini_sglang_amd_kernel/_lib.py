@@ -36,6 +36,10 @@ SIGNATURES = {
         ctypes.c_int,
         [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i64, _i64, _i64, _i64, _i64, _i64,
          _i64, _i64, _i64, _f32, _i32, _i32, _i32, _i32, _vp]),
+    "msgl_build_attention_metadata": (
+        ctypes.c_int,
+        [_vp, _i64, _i64, _i64, _vp, _vp, _vp, _i64, _vp, _vp, _i64, _vp, _vp, _vp, _i64, _vp,
+         _i32, _vp]),
 }
 
 MSGL_DTYPE_BF16 = 0
