@@ -259,6 +259,60 @@ def run_metadata_build(dev, steps: int, warmup: int, cpu_baseline: bool):
     return rows_out
 
 
+def run_norm_rope_store(dev, steps: int, warmup: int, cpu_baseline: bool):
+    """Fused q/k RMSNorm + rotary embedding + KV-store at the token counts of shape 3 (4096 new
+    tokens) and shape 2 (64), 32 q / 8 kv heads of 128.  Every element of q, k, v is read once
+    and written once: 2 * (n_q + 2 n_kv) * d * 2 bytes per token + 8 (position, slot)."""
+    import numpy as np
+    import torch
+
+    from mini_sglang_amd_kernel import qk_norm_rope_store
+
+    n_q, n_kv, d = 32, 8, 128
+    rows_out = []
+    for name, L in (("shape3_new_tokens", 4096), ("shape2_new_tokens", 64)):
+        g = torch.Generator().manual_seed(0x5EED0200 + L)
+        mk = lambda *s: torch.randn(*s, generator=g).to(torch.bfloat16)
+        q, k, v = mk(L, n_q, d), mk(L, n_kv, d), mk(L, n_kv, d)
+        qw, kw = (1 + 0.1 * torch.randn(d, generator=g)).to(torch.bfloat16), (1 + 0.1 * torch.randn(d, generator=g)).to(torch.bfloat16)
+        slots = 2 * L + 64
+        pos = torch.randint(0, 16384, (L,), generator=g, dtype=torch.int32)
+        loc = torch.randperm(slots, generator=g)[:L].to(torch.int32)
+        kc, vc = torch.zeros(slots, n_kv, d, dtype=torch.bfloat16), torch.zeros(slots, n_kv, d, dtype=torch.bfloat16)
+        dq, dk, dv, dqw, dkw, dpos, dloc, dkc, dvc = (t.to(dev) for t in (q, k, v, qw, kw, pos, loc, kc, vc))
+
+        def step():
+            return qk_norm_rope_store(dq, dk, dv, dqw, dkw, dpos, dloc, dkc, dvc, eps=1e-6, rope_base=1e6)
+
+        out = step()
+        torch.cuda.synchronize()
+        mean_ms, per, _ = time_steps(step, steps, warmup)
+        abytes = L * (2 * (n_q + 2 * n_kv) * d * 2 + 8)
+        row = {"sizes": name, "tokens": L, "us_mean": mean_ms * 1e3, "us_min": min(per) * 1e3,
+               "algorithmic_bytes": abytes, "achieved_GBps": abytes / (mean_ms * 1e-3) / 1e9,
+               "hbm_frac": abytes / (mean_ms * 1e-3) / HBM_PEAK}
+        if cpu_baseline:
+            from oracle import qk_norm_rope_oracle as qo  # checker and CPU baseline only
+
+            n = min(L, 512)
+            f = lambda t: t.float().numpy()
+            t1 = time.perf_counter()
+            wq, wkc, wvc = qo.qk_norm_rope_store(f(q[:n]), f(k[:n]), f(v[:n]), f(qw), f(kw), pos[:n].numpy(),
+                                                 loc[:n].numpy(), f(kc), f(vc), 1e-6, 1e6)
+            cpu_s = time.perf_counter() - t1
+            row["cpu_port_GBps"] = n * (2 * (n_q + 2 * n_kv) * d * 2 + 8) / cpu_s / 1e9
+            row["cpu_sample"] = f"first {n} tokens, numpy port, 1 core"
+            dq_err = (out[:n].float().cpu().numpy() - wq)
+            row["q_max_abs_err"] = float(np.abs(dq_err).max())
+            row["v_rows_bit_exact"] = bool(np.array_equal(dvc.float().cpu().numpy()[loc[:n].numpy()],
+                                                          wvc[loc[:n].numpy()]))
+        log(f"[norm+rope+store] {name}: {row['us_mean']:.1f} us mean ({row['us_min']:.1f} min)  "
+            f"{row['achieved_GBps']:.0f} GB/s ({row['hbm_frac']*100:.1f}% of hbm peak)  "
+            f"cpu {row.get('cpu_port_GBps', float('nan')):.3f} GB/s  err {row.get('q_max_abs_err')}")
+        rows_out.append(row)
+    return rows_out
+
+
 def mfma_rate_probe():
     """Sustained v_mfma_f32_32x32x16_bf16 rate of the whole chip on register-resident operands,
     nothing else running: all-zero operands and N(0,1) operands that change every instruction.
@@ -300,7 +354,8 @@ def main():
                     help="also run one device-to-device copy of this many MiB (a kernel of "
                          "known traffic that calibrates rocprofv3 FETCH_SIZE / WRITE_SIZE)")
     ap.add_argument("--no-metadata", action="store_true",
-                    help="skip the on-device metadata build (slot table -> CSR arrays) figures")
+                    help="skip the figures of the kernels either side of the path: on-device metadata "
+                         "build (slot table -> CSR arrays) and fused q/k norm + rope + KV-store")
     ap.add_argument("--no-mfma-probe", action="store_true",
                     help="skip the measurement of the matrix pipe's sustained rate on zero and "
                          "on random operands (the power-limited ceiling the prefill figure is "
@@ -401,6 +456,8 @@ def main():
         if not args.no_mfma_probe:
             result["prefill"]["mfma_rate_probe"] = mfma_rate_probe()
     if not args.no_metadata:
+        result["qk_norm_rope_store"] = run_norm_rope_store(dev, args.steps, args.warmup,
+                                                           not args.no_cpu_baseline)
         result["metadata_build"] = run_metadata_build(dev, args.steps, args.warmup,
                                                       not args.no_cpu_baseline)
     result["all_configs"] = rows

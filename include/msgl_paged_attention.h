@@ -176,6 +176,30 @@ MSGL_API int msgl_build_attention_metadata(const int32_t* page_table, int64_t ta
                                   int32_t max_kv_splits, void* stream);
 
 /*
+ * qk_norm_rope_store -- replaces the chain in front of the attention call in the reference's
+ * Qwen3 attention layer (mini_sglang_mlx/models/qwen3.py:60-68) together with the store that
+ * AttnBackend.forward does first (mini_sglang_mlx/attention/backend.py:139):
+ *     q = q_norm(q); k = k_norm(k)               per-head RMSNorm, weights (head_dim,)
+ *     q = rope(q, positions); k = rope(k, positions)   rotate-half form, rotary_dim = head_dim
+ *     k_cache[out_loc[t]] = k[t]; v_cache[out_loc[t]] = v[t]
+ * in one pass over q, k, v.  q / k / v are (n_tokens, heads, head_dim) bf16 with the two inner
+ * dimensions contiguous and leading strides `*_stride0` in elements (views into a fused QKV
+ * projection are fine); q_out is contiguous (n_tokens, num_q_heads, head_dim).  positions and
+ * out_loc are int32 [n_tokens]; out_loc values must be unique and inside [0, num_slots).
+ * v is copied bit for bit.  head_dim 128 or 256, all pointers 16-byte aligned, strides
+ * multiples of 8 elements.  Attention is then called on q_out WITHOUT another store.
+ */
+MSGL_API int msgl_qk_norm_rope_store(const void* q, const void* k, const void* v,
+                            int64_t q_stride0, int64_t k_stride0, int64_t v_stride0,
+                            const void* q_weight, const void* k_weight,
+                            const int32_t* positions, const int32_t* out_loc,
+                            void* q_out, void* k_cache, void* v_cache,
+                            int64_t k_cache_stride0, int64_t v_cache_stride0, int64_t num_slots,
+                            int64_t n_tokens, int64_t num_q_heads, int64_t num_kv_heads,
+                            int64_t head_dim, float rms_norm_eps, float rope_base,
+                            int32_t dtype, void* stream);
+
+/*
  * Tuning knobs, for benchmarking only (0 = built-in heuristic).  Process-wide,
  * read at launch time; not part of the reference surface.
  *   MSGL_TUNE_SEGMENTS       segments the split-K kernel cuts the visible token stream into

@@ -317,4 +317,53 @@ int msgl_build_attention_metadata(const int32_t* page_table, int64_t table_strid
   return msgl::launch_build_metadata(a, static_cast<hipStream_t>(stream));
 }
 
+int msgl_qk_norm_rope_store(const void* q, const void* k, const void* v, int64_t q_stride0,
+                            int64_t k_stride0, int64_t v_stride0, const void* q_weight,
+                            const void* k_weight, const int32_t* positions,
+                            const int32_t* out_loc, void* q_out, void* k_cache, void* v_cache,
+                            int64_t k_cache_stride0, int64_t v_cache_stride0, int64_t num_slots,
+                            int64_t n_tokens, int64_t num_q_heads, int64_t num_kv_heads,
+                            int64_t head_dim, float rms_norm_eps, float rope_base, int32_t dtype,
+                            void* stream) {
+  if (head_dim != 128 && head_dim != 256) return MSGL_ERR_HEAD_DIM;
+  if (dtype != MSGL_DTYPE_BF16) return MSGL_ERR_DTYPE;
+  if (n_tokens < 0 || num_q_heads <= 0 || num_kv_heads <= 0 || num_slots < 0) return MSGL_ERR_SHAPE;
+  if (!(rope_base > 1.0f) || !(rms_norm_eps >= 0.0f)) return MSGL_ERR_SHAPE;
+  if (q_stride0 < num_q_heads * head_dim || k_stride0 < num_kv_heads * head_dim ||
+      v_stride0 < num_kv_heads * head_dim || k_cache_stride0 < num_kv_heads * head_dim ||
+      v_cache_stride0 < num_kv_heads * head_dim)
+    return MSGL_ERR_SHAPE;
+  if (n_tokens == 0) return MSGL_OK;
+  if (!q || !k || !v || !q_weight || !k_weight || !positions || !out_loc || !q_out || !k_cache ||
+      !v_cache)
+    return MSGL_ERR_NULL_POINTER;
+  if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(q_weight) ||
+      !aligned16(k_weight) || !aligned16(q_out) || !aligned16(k_cache) || !aligned16(v_cache) ||
+      q_stride0 % 8 || k_stride0 % 8 || v_stride0 % 8 || k_cache_stride0 % 8 || v_cache_stride0 % 8)
+    return MSGL_ERR_ALIGNMENT;
+  msgl::NormRopeArgs a{};
+  a.q = q;
+  a.k = k;
+  a.v = v;
+  a.q_weight = q_weight;
+  a.k_weight = k_weight;
+  a.positions = positions;
+  a.out_loc = out_loc;
+  a.q_out = q_out;
+  a.k_cache = k_cache;
+  a.v_cache = v_cache;
+  a.q_stride0 = q_stride0;
+  a.k_stride0 = k_stride0;
+  a.v_stride0 = v_stride0;
+  a.kc_stride0 = k_cache_stride0;
+  a.vc_stride0 = v_cache_stride0;
+  a.n_tokens = n_tokens;
+  a.n_q = num_q_heads;
+  a.n_kv = num_kv_heads;
+  a.head_dim = head_dim;
+  a.eps = rms_norm_eps;
+  a.rope_base = rope_base;
+  return msgl::launch_qk_norm_rope_store(a, static_cast<hipStream_t>(stream));
+}
+
 }  // extern "C"

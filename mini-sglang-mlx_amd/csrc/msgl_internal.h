@@ -91,6 +91,24 @@ struct MetadataArgs {
 constexpr int64_t kMetadataMaxBatch = 8000;
 int launch_build_metadata(const MetadataArgs& a, hipStream_t stream);
 
+// ---- qk_norm_rope_store.hip ----------------------------------------------------------
+struct NormRopeArgs {
+  const void* q;
+  const void* k;
+  const void* v;
+  const void* q_weight;
+  const void* k_weight;
+  const int32_t* positions;
+  const int32_t* out_loc;
+  void* q_out;
+  void* k_cache;
+  void* v_cache;
+  int64_t q_stride0, k_stride0, v_stride0, kc_stride0, vc_stride0;  // elements
+  int64_t n_tokens, n_q, n_kv, head_dim;
+  float eps, rope_base;
+};
+int launch_qk_norm_rope_store(const NormRopeArgs& a, hipStream_t stream);
+
 inline int check_launch() { return hipGetLastError() == hipSuccess ? MSGL_OK : MSGL_ERR_LAUNCH; }
 
 }  // namespace msgl

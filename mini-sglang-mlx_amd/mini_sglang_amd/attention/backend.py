@@ -16,7 +16,7 @@ from typing import List, Optional, Sequence
 import torch
 
 from mini_sglang_amd_kernel import (build_attention_metadata, paged_decode_attention,
-                                    paged_prefill_attention)
+                                    paged_prefill_attention, qk_norm_rope_store)
 
 MAX_KV_SPLITS = 32
 
@@ -86,7 +86,10 @@ class AttnBackend:
         self.kvcache.store_kv(k, v, batch.out_loc, layer_id)
         k_cache = self.kvcache.k_cache(layer_id)
         v_cache = self.kvcache.v_cache(layer_id)
+        return self._attend(q, k_cache, v_cache, metadata, is_cross_attention, sliding_window_size)
 
+    def _attend(self, q, k_cache, v_cache, metadata, is_cross_attention: bool,
+                sliding_window_size: int) -> torch.Tensor:
         if isinstance(metadata, PrefillMetadata):
             return paged_prefill_attention(
                 q, k_cache, v_cache, metadata.qo_indptr, metadata.kv_indptr, metadata.kv_indices,
@@ -101,6 +104,26 @@ class AttnBackend:
         return paged_decode_attention(
             q, k_cache, v_cache, metadata.kv_indptr, metadata.kv_indices, metadata.num_kv_splits,
             sm_scale=self.sm_scale, max_kv_splits=metadata.max_kv_splits)
+
+    def forward_fused_norm_rope(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
+                                q_norm_weight: torch.Tensor, k_norm_weight: torch.Tensor,
+                                layer_id: int, batch, *, rms_norm_eps: float, rope_base: float,
+                                is_cross_attention: bool = False,
+                                sliding_window_size: int = 0) -> torch.Tensor:
+        """``forward`` for a Qwen3-style layer that hands over the raw projections: q/k RMSNorm,
+        rotary embedding at ``batch.attn_metadata.positions`` and the KV-store run as one kernel
+        (the reference does them as four array ops plus the store, models/qwen3.py:60-68 and
+        backend.py:139), then attention runs on the pool without storing again."""
+        assert sliding_window_size >= 0, (
+            f"sliding_window_size must be >= 0, got {sliding_window_size}"
+        )
+        metadata = batch.attn_metadata
+        k_cache = self.kvcache.k_cache(layer_id)
+        v_cache = self.kvcache.v_cache(layer_id)
+        q = qk_norm_rope_store(q, k, v, q_norm_weight, k_norm_weight, metadata.positions,
+                               batch.out_loc, k_cache, v_cache, eps=rms_norm_eps,
+                               rope_base=rope_base)
+        return self._attend(q, k_cache, v_cache, metadata, is_cross_attention, sliding_window_size)
 
     def store_kv_only(self, k: torch.Tensor, v: torch.Tensor, out_loc: torch.Tensor,
                       layer_id: int) -> None:

@@ -21,7 +21,7 @@ import torch
 from . import _lib
 
 __all__ = ["store_kv_cache", "paged_decode_attention", "paged_prefill_attention",
-           "build_attention_metadata"]
+           "build_attention_metadata", "qk_norm_rope_store"]
 
 _DTYPE_CODE = {torch.bfloat16: _lib.MSGL_DTYPE_BF16, torch.float16: _lib.MSGL_DTYPE_F16}
 
@@ -321,3 +321,56 @@ def build_attention_metadata(page_table: torch.Tensor, table_rows: torch.Tensor,
         total_q, out["num_kv_splits"].data_ptr(), int(max_kv_splits), _stream_ptr(stream, dev))
     _check_rc(op, rc)
     return out
+
+
+def _heads_stride0(op: str, t: torch.Tensor, name: str) -> int:
+    if t.dim() != 3:
+        _fail(op, f"{name} must be 3D (tokens, heads, head_dim)")
+    if t.stride(2) != 1 or t.stride(1) != t.shape[2]:
+        _fail(op, f"{name} must be contiguous in its (heads, head_dim) dimensions")
+    return t.stride(0) if t.shape[0] > 1 else t.shape[1] * t.shape[2]
+
+
+def qk_norm_rope_store(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, q_weight: torch.Tensor,
+                       k_weight: torch.Tensor, positions: torch.Tensor, out_loc: torch.Tensor,
+                       k_cache: torch.Tensor, v_cache: torch.Tensor, *, eps: float,
+                       rope_base: float, stream=None) -> torch.Tensor:
+    """Per-head RMSNorm of q and k, rotary embedding of both at ``positions``, and the store of
+    the new k and v rows at ``out_loc``, in one pass; returns the rotated q.
+
+    One call for ``q_norm`` / ``k_norm`` / ``rope`` / ``rope`` of the reference's Qwen3 attention
+    layer (mini_sglang_mlx/models/qwen3.py:60-68) plus the store that ``AttnBackend.forward``
+    does first (attention/backend.py:139).  Attention then runs on the result with no further
+    store.  q / k / v may be strided views (tokens, heads, head_dim) of a fused projection.
+    """
+    op = "qk_norm_rope_store"
+    dev = _require_device(op, q, k, v, q_weight, k_weight, positions, out_loc, k_cache, v_cache)
+    qs, ks, vs = (_heads_stride0(op, t, n) for t, n in ((q, "q"), (k, "k"), (v, "v")))
+    n_tokens, n_q, d = q.shape
+    n_kv = k.shape[1]
+    if d not in (128, 256):
+        _fail(op, "head_dim must be 128 or 256")
+    if tuple(k.shape) != (n_tokens, n_kv, d) or tuple(v.shape) != (n_tokens, n_kv, d):
+        _fail(op, "k and v shape must be (tokens, num_kv_heads, head_dim)")
+    if k_cache.dim() != 3 or tuple(k_cache.shape[1:]) != (n_kv, d) or k_cache.shape != v_cache.shape:
+        _fail(op, "k_cache and v_cache must be (num_pages, num_kv_heads, head_dim)")
+    for t, name in ((q, "q"), (k, "k"), (v, "v"), (k_cache, "k_cache"), (v_cache, "v_cache"),
+                    (q_weight, "q_weight"), (k_weight, "k_weight")):
+        if t.dtype != torch.bfloat16:
+            _fail(op, f"{name} must be bfloat16")
+    if tuple(q_weight.shape) != (d,) or tuple(k_weight.shape) != (d,):
+        _fail(op, "q_weight and k_weight must be (head_dim,)")
+    positions = _int32_1d(op, positions, "positions")
+    out_loc = _int32_1d(op, out_loc, "out_loc")
+    if positions.shape[0] != n_tokens or out_loc.shape[0] != n_tokens:
+        _fail(op, "positions and out_loc length must match q length")
+    q_out = torch.empty((n_tokens, n_q, d), dtype=q.dtype, device=dev)
+    rc = _lib.load().msgl_qk_norm_rope_store(
+        q.data_ptr(), k.data_ptr(), v.data_ptr(), qs, ks, vs, q_weight.contiguous().data_ptr(),
+        k_weight.contiguous().data_ptr(), positions.data_ptr(), out_loc.data_ptr(),
+        q_out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+        _pool_stride0(op, k_cache, "k_cache"), _pool_stride0(op, v_cache, "v_cache"),
+        k_cache.shape[0], n_tokens, n_q, n_kv, d, float(eps), float(rope_base),
+        _lib.MSGL_DTYPE_BF16, _stream_ptr(stream, dev))
+    _check_rc(op, rc)
+    return q_out

@@ -40,6 +40,10 @@ SIGNATURES = {
         ctypes.c_int,
         [_vp, _i64, _i64, _i64, _vp, _vp, _vp, _i64, _vp, _vp, _i64, _vp, _vp, _vp, _i64, _vp,
          _i32, _vp]),
+    "msgl_qk_norm_rope_store": (
+        ctypes.c_int,
+        [_vp, _vp, _vp, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64,
+         _i64, _i64, _i64, _i64, _f32, _f32, _i32, _vp]),
 }
 
 MSGL_DTYPE_BF16 = 0
