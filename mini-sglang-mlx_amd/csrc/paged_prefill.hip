@@ -44,6 +44,7 @@ namespace {
 #endif
 
 typedef short s16x4_t __attribute__((ext_vector_type(4)));
+constexpr bf16x2_t kOnes = {(__bf16)1.0f, (__bf16)1.0f};
 #define MSGL_LDS_PTR(T, p) ((__attribute__((address_space(3))) T*)(p))
 
 constexpr int kUnitRows = 4;                 // rows moved by one LDS-direct load
@@ -167,6 +168,14 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
     for (int ks = 0; ks < KSTEPS; ++ks) {
       u32x4_t raw = {0u, 0u, 0u, 0u};
       if (valid) raw = ld_global_b128(p.q + off + ks * 16 + h * 8);
+      // q carries the softmax scale (and log2 e) from here on: scores leave the MFMA ready
+      // for exp2, at the price of one more bf16 rounding of q
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float lo = __builtin_bit_cast(float, raw[e] << 16) * p.scale_log2e;
+        const float hi = __builtin_bit_cast(float, raw[e] & 0xffff0000u) * p.scale_log2e;
+        raw[e] = pack_bf16x2(lo, hi);
+      }
       qreg[rt][ks] = as_bf16x8(raw);
     }
     const int qpos = prefix + qi;
@@ -198,10 +207,15 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
 #pragma unroll
       for (int i = 0; i < 16; ++i) oacc[dt][rt][i] = 0.f;
   float m_run[RT], l_run[RT];
+  // The score MFMAs start from -m (the running row max, 0 while there is none) instead of
+  // from 0, so a half tile's scores arrive already shifted and go straight into exp2.
+  f32x16_t s_init[RT];
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
     m_run[rt] = kNegInf;
     l_run[rt] = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) s_init[rt][i] = 0.f;
   }
 
   // ---- moving a tile: wave w owns units w*UPW .. w*UPW+UPW-1; in a unit, lane l fetches
@@ -216,7 +230,7 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
   const int unit_key = w * UPW + 16 * (lane >> 4);  // + i for unit i of this wave
   auto row_offset = [&](int32_t slot_id, uint32_t row_bytes) -> OffT {
     if constexpr (WIDE) return (uint64_t)(uint32_t)slot_id * row_bytes + chunk_off;
-    else return (uint32_t)slot_id * row_bytes + chunk_off;
+    else return __umul24((uint32_t)slot_id, row_bytes) + chunk_off;  // both below 2^24 here
   };
   int32_t slot[UPW];  // slot ids of the tile whose K moves next, fetched one iteration ahead
   OffT k_off[UPW];    // K row offsets of that tile
@@ -307,15 +321,11 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
       }
     }
   };
-  // Softmax state of one half tile, decided as soon as its scores exist:
-  //   mul    factor still to be applied to the scores: the softmax scale on interior halves
-  //          (raw scores; max commutes with a positive scale), 1 on boundary halves, which
-  //          are scaled and masked in place
-  //   m_safe the (lazy) running row max the half's exponentials are taken against
-  //   alpha  exp2(previous max - m_safe): what O and l must be multiplied by first
+  // Softmax state of one half tile, decided as soon as its scores exist: alpha = exp2(previous
+  // running max - new one), what O and l must be multiplied by before this half is added.
+  // The scores themselves are left shifted by the new max, ready for exp2.
   struct Stats {
-    float mul;
-    float m_safe[RT], alpha[RT];
+    float alpha[RT];
   };
   auto mask_in_place = [&](Scores& sc, int base) {
 #pragma unroll
@@ -323,8 +333,7 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         const int key = base + 8 * (i >> 2) + 4 * h + (i & 3);
-        const float x = sc.s[rt][i] * p.scale_log2e;
-        sc.s[rt][i] = (key < row_lo[rt] || key > row_hi[rt]) ? kNegInf : x;
+        if (key < row_lo[rt] || key > row_hi[rt]) sc.s[rt][i] = kNegInf;
       }
   };
   auto lane_max = [&](const Scores& sc, float (&mx)[RT]) {
@@ -336,18 +345,29 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
       mx[rt] = m;
     }
   };
-  auto decide = [&](const float (&mx)[RT], Stats& st) {
+  // mx: per-lane max of scores that are relative to the running max (to 0 if there is none
+  // yet).  The running max only moves when it grows by more than kLazy; then (rarely) the
+  // scores are shifted once more and the MFMA start values are refreshed.
+  auto decide = [&](Scores& sc, const float (&mx)[RT], Stats& st) {
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
-      const float m = wave_max_xor(mx[rt] * st.mul, 32);
       const float m_old = m_run[rt];
-      const float m_new = fmaxf(m_old, m);
+      const float ref = (m_old == kNegInf) ? 0.f : m_old;
+      const float cand = ref + wave_max_xor(mx[rt], 32);
+      const float m_new = fmaxf(m_old, cand);
       const float m_use = (m_new - m_old > kLazy) ? m_new : m_old;
-      st.m_safe[rt] = (m_use == kNegInf) ? 0.f : m_use;
-      st.alpha[rt] = fast_exp2(m_old - st.m_safe[rt]);
+      const float m_safe = (m_use == kNegInf) ? 0.f : m_use;
+      const float shift = m_safe - ref;
+      st.alpha[rt] = fast_exp2(m_old - m_safe);
       m_run[rt] = m_use;
-      pin(st.m_safe[rt]);
       pin(st.alpha[rt]);
+      if (__any(shift != 0.f)) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          sc.s[rt][i] -= shift;
+          s_init[rt][i] = -m_safe;
+        }
+      }
     }
   };
   // One pipeline step over half tiles i-1, i, i+1.  The matrix pipe computes the scores of
@@ -374,10 +394,9 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
       for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
         for (int i = first; i < first + 8; ++i) {
-          float e = fast_exp2(__builtin_fmaf(cur.s[rt][i], st_cur.mul, -st_cur.m_safe[rt]));
+          float e = fast_exp2(cur.s[rt][i]);
           pin(e);
           cur.s[rt][i] = e;
-          psum[rt] += e;
         }
     };
     auto pack_slice = [&](int u) {
@@ -389,6 +408,8 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
           uint32_t pw = pack_bf16x2(cur.s[rt][8 * u + 2 * j], cur.s[rt][8 * u + 2 * j + 1]);
           pin(pw);
           pk[j] = pw;
+          // row sum of the rounded weights, the ones that multiply V
+          psum[rt] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, pw), kOnes, psum[rt], false);
         }
         pb_cur[rt][u] = as_bf16x8(pk);
       }
@@ -398,7 +419,8 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
       for (int e = 0; e < 4; ++e)
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt)
-          nxt.s[rt] = mfma_32x32x16(ops[e], qreg[rt][first + e], nxt.s[rt]);
+          nxt.s[rt] = mfma_32x32x16(ops[e], qreg[rt][first + e],
+                                    (first + e == 0) ? s_init[rt] : nxt.s[rt]);
     };
     auto pv_slice = [&](int u, const bf16x8_t (&ops)[4]) {  // 16 keys, all four dim tiles
 #pragma unroll
@@ -409,11 +431,7 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
     bf16x8_t ops_a[4], ops_b[4];
     // slice 0
 #pragma unroll
-    for (int rt = 0; rt < RT; ++rt) {
-      psum[rt] = 0.f;
-#pragma unroll
-      for (int i = 0; i < 16; ++i) nxt.s[rt][i] = 0.f;
-    }
+    for (int rt = 0; rt < RT; ++rt) psum[rt] = 0.f;
 #pragma unroll
     for (int e = 0; e < 4; ++e) ops_a[e] = k_operand(ks, 4 + e);
     qk_slice(0, kops);
@@ -430,13 +448,11 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
     side(1);
     MSGL_TICK(8 + 4 * prof_half + 1);
     __builtin_amdgcn_sched_barrier(0);
-    st_nxt.mul = p.scale_log2e;
-    if (mask_nxt) {  // boundary half: scale and mask in place
+    if (mask_nxt) {  // boundary half: mask in place
       // the empty volatile statement keeps this a branch: turned into selects it would put
-      // 64 extra VALU instructions into every half tile
+      // extra VALU instructions into every half tile
       asm volatile("" ::: "memory");
       mask_in_place(nxt, nxt_base);
-      st_nxt.mul = 1.0f;
     }
     // slice 2
 #pragma unroll
@@ -456,7 +472,7 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
     pv_slice(1, ops_a);
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) l_run[rt] = l_run[rt] * st_cur.alpha[rt] + psum[rt];
-    decide(mx, st_nxt);
+    decide(nxt, mx, st_nxt);
     side(3);
     MSGL_TICK(8 + 4 * prof_half + 3);
     __builtin_amdgcn_sched_barrier(0);
@@ -468,9 +484,8 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
   // third K and V stages.  Every move is unconditional (tiles past the end clamp to the last
   // key and are fully masked).  A wave waits for its own moves at the end of the iteration,
   // then the workgroup barrier publishes them: one barrier per tile.
-  const bool general_scale = p.scale_log2e <= 0.f;  // fast path needs a positive scale
   auto needs_mask = [&](int base) {  // some row of this wave sees only part of keys base .. base+31
-    return general_scale || (base < w_lo_max) || (base + 31 > w_hi_min);
+    return (base < w_lo_max) || (base + 31 > w_hi_min);
   };
   if (n_tiles > 0) {
     slot_load(k_lo);
@@ -490,21 +505,15 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
     Stats st_a, st_b;
     bf16x8_t pb_a[RT][2], pb_b[RT][2];
     qk_half(0, 0, sa);
-    st_a.mul = p.scale_log2e;
-    if (needs_mask(k_lo)) {
-      mask_in_place(sa, k_lo);
-      st_a.mul = 1.0f;
-    }
+    if (needs_mask(k_lo)) mask_in_place(sa, k_lo);
     {
       float mx[RT];
       lane_max(sa, mx);
-      decide(mx, st_a);
+      decide(sa, mx, st_a);
     }
-    st_b.mul = 1.0f;
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
       st_b.alpha[rt] = 1.0f;
-      st_b.m_safe[rt] = 0.f;
 #pragma unroll
       for (int u = 0; u < 2; ++u) pb_b[rt][u] = as_bf16x8(u32x4_t{0u, 0u, 0u, 0u});
     }

@@ -61,8 +61,11 @@ inline int make_prefill_params(const PrefillArgs& a, PrefillParams& p, int64_t& 
   if (n_blocks > 0x7fffffffLL) return MSGL_ERR_SHAPE;
   p.n_qblk = (int32_t)n_qblk;
   p.n_pairs = (int32_t)n_pairs;
+  // narrow offsets: slot * row_bytes fits 32 bits and both factors fit 24 bits (one
+  // full-rate 24-bit multiply per row)
   wide = (uint64_t)a.num_slots * (uint64_t)a.k_stride0 * 2u >= (1ull << 32) ||
-         (uint64_t)a.num_slots * (uint64_t)a.v_stride0 * 2u >= (1ull << 32);
+         (uint64_t)a.num_slots * (uint64_t)a.v_stride0 * 2u >= (1ull << 32) ||
+         a.num_slots >= (1 << 24) || a.k_stride0 * 2 >= (1 << 24) || a.v_stride0 * 2 >= (1 << 24);
   return MSGL_OK;
 }
 
