@@ -313,6 +313,61 @@ def run_norm_rope_store(dev, steps: int, warmup: int, cpu_baseline: bool):
     return rows_out
 
 
+def run_gdn_state(dev, steps: int, warmup: int, cpu_baseline: bool):
+    """Gated delta-rule state kernel at the reference's benchmark sizes (hk 16, hv 32,
+    dk = dv = 128; test_and_bench/gdn_state.py:33-48): decode of 8 requests (HBM-bound, the
+    fp32 state of every (request, head) read and written once) and a 1024-token prefill (a
+    serial chain per state row)."""
+    import numpy as np
+    import torch
+
+    from mini_sglang_amd_kernel import gdn_state_inplace
+
+    hk, hv, d = 16, 32, 128
+    rows_out = []
+    for name, lengths, single in (("decode_batch8", [1] * 8, True), ("decode_batch64", [1] * 64, True),
+                                  ("prefill_1024", [1024], False)):
+        g = torch.Generator().manual_seed(0x5EED0300 + len(lengths))
+        T, B = sum(lengths), len(lengths)
+        bf = lambda *s: (0.05 * torch.randn(*s, generator=g)).to(torch.bfloat16)
+        sg = lambda *s: torch.sigmoid(torch.randn(*s, generator=g)).to(torch.bfloat16)
+        q, k, v, gg, beta = bf(T, hk, d), bf(T, hk, d), bf(T, hv, d), sg(T, hv), sg(T, hv)
+        state = 0.05 * torch.randn(B + 1, hv, d, d, generator=g)
+        slots = torch.arange(B, dtype=torch.int32)
+        ip = torch.tensor([0] + list(np.cumsum(lengths)), dtype=torch.int32)
+        dq, dk, dv, dg, db, dst, dsl, dip = (t.to(dev) for t in (q, k, v, gg, beta, state, slots, ip))
+
+        def step():
+            return gdn_state_inplace(dq, dk, dv, dg, db, dst, dsl, dip, single_token_mode=single)
+
+        step()
+        torch.cuda.synchronize()
+        mean_ms, per, _ = time_steps(step, steps, warmup)
+        state_bytes = 2 * B * hv * d * d * 4
+        io_bytes = T * (2 * hk * d * 2 + 2 * hv * d * 2 + 2 * hv * 2)
+        row = {"sizes": name, "tokens": T, "batch": B, "us_mean": mean_ms * 1e3, "us_min": min(per) * 1e3,
+               "algorithmic_bytes": state_bytes + io_bytes,
+               "achieved_GBps": (state_bytes + io_bytes) / (mean_ms * 1e-3) / 1e9,
+               "tokens_per_s": T / (mean_ms * 1e-3)}
+        if cpu_baseline:
+            from oracle import gdn_state_oracle as go  # checker and CPU baseline only
+
+            n = min(T, 8)
+            f = lambda t: t.float().numpy()
+            nb = B if single else 1
+            t1 = time.perf_counter()
+            go.gdn_state_inplace(f(q[:n]), f(k[:n]), f(v[:n]), f(gg[:n]), f(beta[:n]), state.numpy(),
+                                 slots[:min(nb, n)].numpy(), None if single else np.array([0, n], np.int32),
+                                 single_token_mode=single)
+            row["cpu_port_tokens_per_s"] = n / (time.perf_counter() - t1)
+            row["cpu_sample"] = f"first {n} tokens, numpy float64 port, 1 core"
+        log(f"[gdn_state] {name}: {row['us_mean']:.1f} us mean ({row['us_min']:.1f} min)  "
+            f"{row['achieved_GBps']:.0f} GB/s  {row['tokens_per_s']:.3g} tokens/s  "
+            f"cpu {row.get('cpu_port_tokens_per_s', float('nan')):.3g} tokens/s")
+        rows_out.append(row)
+    return rows_out
+
+
 def mfma_rate_probe():
     """Sustained v_mfma_f32_32x32x16_bf16 rate of the whole chip on register-resident operands,
     nothing else running: all-zero operands and N(0,1) operands that change every instruction.
@@ -458,6 +513,8 @@ def main():
     if not args.no_metadata:
         result["qk_norm_rope_store"] = run_norm_rope_store(dev, args.steps, args.warmup,
                                                            not args.no_cpu_baseline)
+        result["gdn_state_inplace"] = run_gdn_state(dev, args.steps, args.warmup,
+                                                    not args.no_cpu_baseline)
         result["metadata_build"] = run_metadata_build(dev, args.steps, args.warmup,
                                                       not args.no_cpu_baseline)
     result["all_configs"] = rows

@@ -57,6 +57,7 @@ extern "C" {
 #define MSGL_ERR_ALIGNMENT (-10)        /* pointer or stride not aligned for the vector width used */
 #define MSGL_ERR_LAUNCH (-11)           /* the HIP runtime refused a launch (hipGetLastError) */
 #define MSGL_ERR_HEAD_DIM_MULT4 (-12)   /* store: head_dim is not a multiple of 4 */
+#define MSGL_ERR_GDN_DIMS (-13)         /* gdn_state_inplace: dk and dv must both be 128 */
 
 /* Library version: major*10000 + minor*100 + patch. */
 MSGL_API int msgl_version(void);
@@ -200,6 +201,28 @@ MSGL_API int msgl_qk_norm_rope_store(const void* q, const void* k, const void* v
                             int32_t dtype, void* stream);
 
 /*
+ * gdn_state_inplace -- replaces mini_sglang_mlx::gdn_state_inplace
+ * (mini-sglang-mlx-kernel/csrc/gdn_state.cpp:87-183, kernel gdn_state.metal:14-99), the gated
+ * delta-rule recurrence of the hybrid (Qwen3.5) layers with a slot-indexed state:
+ * for request b, state S = state[slot_ids[b]] of shape (hv, dv, dk), and each of its tokens t
+ * in order
+ *     S *= g[t, h];  delta = (v[t, h, :] - S[h] k[t, h / (hv / hk)]) * beta[t, h]
+ *     S[h] += outer(delta, k[t, h / (hv / hk)]);  y[t, h, :] = S[h] q[t, h / (hv / hk)]
+ * q, k: (tokens, hk, 128) bf16; v, y: (tokens, hv, 128) bf16; g, beta: (tokens, hv) bf16
+ * contiguous; state: (num_slots, hv, 128, 128) fp32, updated in place; slot_ids int32 [batch]
+ * (distinct, inside [0, num_slots)); qo_indptr int32 [batch + 1], the token range of each
+ * request, ignored in single_token_mode (one token per request, token b belongs to request
+ * b; the reference's decode mode).  *_stride0: leading strides in elements (the reference
+ * uses q's for k as well, gdn_state.cpp:163-164; here both are taken).  hv % hk == 0.
+ */
+MSGL_API int msgl_gdn_state_inplace(const void* q, const void* k, const void* v, const void* g,
+                           const void* beta, void* state, const int32_t* slot_ids,
+                           const int32_t* qo_indptr, void* y, int64_t tokens, int64_t batch,
+                           int64_t hk, int64_t hv, int64_t dk, int64_t dv, int64_t num_slots,
+                           int64_t state_stride0, int64_t q_stride0, int64_t k_stride0,
+                           int64_t v_stride0, int32_t single_token_mode, void* stream);
+
+/*
  * Tuning knobs, for benchmarking only (0 = built-in heuristic).  Process-wide,
  * read at launch time; not part of the reference surface.
  *   MSGL_TUNE_SEGMENTS       segments the split-K kernel cuts the visible token stream into
@@ -208,12 +231,15 @@ MSGL_API int msgl_qk_norm_rope_store(const void* q, const void* k, const void* v
  *   MSGL_TUNE_PREFILL_VARIANT tiling of the MFMA kernel (0: 8 waves x 32 rows, 1: 4 x 64)
  *   MSGL_TUNE_SPLITKV_WAVES  most waves (adjacent kv heads) per split-K workgroup: 1, 2, 4, 8
  *                            (0 restores the default, 4)
+ *   MSGL_TUNE_GDN_ROWS       state rows per 16-lane group of the gdn_state kernel: 1, 2, 4
+ *                            (0: chosen from the problem size)
  */
 #define MSGL_TUNE_SEGMENTS 0
 #define MSGL_TUNE_MIN_SEGMENT 1
 #define MSGL_TUNE_SMALLQ_MAXCOLS 2
 #define MSGL_TUNE_PREFILL_VARIANT 3
 #define MSGL_TUNE_SPLITKV_WAVES 4
+#define MSGL_TUNE_GDN_ROWS 5
 MSGL_API int msgl_set_tuning(int32_t knob, int64_t value);
 
 #ifdef __cplusplus

@@ -21,7 +21,8 @@ LIB_PATH = os.path.join(LIB_DIR, "libmsgl_paged_attention.so")
 PROBE_SRC = os.path.join(CSRC, "probes", "mfma_rate_probe.hip")
 PROBE_PATH = os.path.join(LIB_DIR, "libmsgl_probes.so")
 SOURCES = ["api.hip", "store_kv_cache.hip", "paged_splitkv.hip", "paged_prefill.hip",
-           "build_metadata.hip", "qk_norm_rope_store.hip"]
+           "build_metadata.hip", "qk_norm_rope_store.hip",
+           "gdn_state.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # Packed fp32 VALU forms are switched off for every device compile on this target.

@@ -68,6 +68,7 @@ const char* msgl_strerror(int code) {
     case MSGL_ERR_ALIGNMENT: return "pointer or stride not aligned to the vector width";
     case MSGL_ERR_LAUNCH: return "HIP kernel launch failed";
     case MSGL_ERR_HEAD_DIM_MULT4: return "head_dim must be a multiple of 4";
+    case MSGL_ERR_GDN_DIMS: return "this specialized kernel requires dk=dv=128";
     default: return "unknown error code";
   }
 }
@@ -75,6 +76,10 @@ const char* msgl_strerror(int code) {
 int msgl_set_tuning(int32_t knob, int64_t value) {
   if (knob == MSGL_TUNE_SPLITKV_WAVES) {
     msgl::splitkv_set_max_waves((int)value);
+    return MSGL_OK;
+  }
+  if (knob == MSGL_TUNE_GDN_ROWS) {
+    msgl::gdn_set_rows((int)value);
     return MSGL_OK;
   }
   if (knob == MSGL_TUNE_PREFILL_VARIANT) {
@@ -364,6 +369,47 @@ int msgl_qk_norm_rope_store(const void* q, const void* k, const void* v, int64_t
   a.eps = rms_norm_eps;
   a.rope_base = rope_base;
   return msgl::launch_qk_norm_rope_store(a, static_cast<hipStream_t>(stream));
+}
+
+int msgl_gdn_state_inplace(const void* q, const void* k, const void* v, const void* g,
+                           const void* beta, void* state, const int32_t* slot_ids,
+                           const int32_t* qo_indptr, void* y, int64_t tokens, int64_t batch,
+                           int64_t hk, int64_t hv, int64_t dk, int64_t dv, int64_t num_slots,
+                           int64_t state_stride0, int64_t q_stride0, int64_t k_stride0,
+                           int64_t v_stride0, int32_t single_token_mode, void* stream) {
+  if (dk != 128 || dv != 128) return MSGL_ERR_GDN_DIMS;  // gdn_state.cpp:80-83
+  if (tokens < 0 || batch < 0 || hk <= 0 || hv <= 0 || num_slots < 0) return MSGL_ERR_SHAPE;
+  if (hv % hk != 0) return MSGL_ERR_HEAD_RATIO;          // gdn_state.cpp:76-79
+  if (single_token_mode && tokens != batch) return MSGL_ERR_SHAPE;  // :107-111
+  if (state_stride0 < hv * dv * dk || q_stride0 < hk * dk || k_stride0 < hk * dk ||
+      v_stride0 < hv * dv)
+    return MSGL_ERR_SHAPE;
+  if (tokens == 0 || batch == 0) return MSGL_OK;
+  if (!q || !k || !v || !g || !beta || !state || !slot_ids || !y) return MSGL_ERR_NULL_POINTER;
+  if (!single_token_mode && !qo_indptr) return MSGL_ERR_NULL_POINTER;
+  if (!aligned16(q) || !aligned16(k) || !aligned16(state) || q_stride0 % 8 || k_stride0 % 8 ||
+      state_stride0 % 4)
+    return MSGL_ERR_ALIGNMENT;
+  msgl::GdnArgs a{};
+  a.q = q;
+  a.k = k;
+  a.v = v;
+  a.g = g;
+  a.beta = beta;
+  a.state = state;
+  a.slot_ids = slot_ids;
+  a.qo_indptr = qo_indptr;
+  a.y = y;
+  a.tokens = tokens;
+  a.batch = batch;
+  a.hk = hk;
+  a.hv = hv;
+  a.state_stride0 = state_stride0;
+  a.q_stride0 = q_stride0;
+  a.k_stride0 = k_stride0;
+  a.v_stride0 = v_stride0;
+  a.single_token_mode = single_token_mode;
+  return msgl::launch_gdn_state(a, static_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

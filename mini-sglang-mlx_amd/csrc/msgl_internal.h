@@ -109,6 +109,25 @@ struct NormRopeArgs {
 };
 int launch_qk_norm_rope_store(const NormRopeArgs& a, hipStream_t stream);
 
+// ---- gdn_state.hip ---------------------------------------------------------------------
+struct GdnArgs {
+  const void* q;
+  const void* k;
+  const void* v;
+  const void* g;
+  const void* beta;
+  void* state;
+  const int32_t* slot_ids;
+  const int32_t* qo_indptr;  // unused in single-token mode
+  void* y;
+  int64_t tokens, batch, hk, hv;
+  int64_t state_stride0, q_stride0, k_stride0, v_stride0;  // elements
+  int32_t single_token_mode;
+};
+int launch_gdn_state(const GdnArgs& a, hipStream_t stream);
+// benchmarking switch: state rows per 16-lane group (1, 2, 4; 0 = chosen from the problem size)
+void gdn_set_rows(int v);
+
 inline int check_launch() { return hipGetLastError() == hipSuccess ? MSGL_OK : MSGL_ERR_LAUNCH; }
 
 }  // namespace msgl

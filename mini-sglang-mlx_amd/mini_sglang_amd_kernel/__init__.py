@@ -21,7 +21,7 @@ import torch
 from . import _lib
 
 __all__ = ["store_kv_cache", "paged_decode_attention", "paged_prefill_attention",
-           "build_attention_metadata", "qk_norm_rope_store"]
+           "build_attention_metadata", "qk_norm_rope_store", "gdn_state_inplace"]
 
 _DTYPE_CODE = {torch.bfloat16: _lib.MSGL_DTYPE_BF16, torch.float16: _lib.MSGL_DTYPE_F16}
 
@@ -374,3 +374,71 @@ def qk_norm_rope_store(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, q_weig
         _lib.MSGL_DTYPE_BF16, _stream_ptr(stream, dev))
     _check_rc(op, rc)
     return q_out
+
+
+def gdn_state_inplace(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Tensor,
+                      beta: torch.Tensor, state: torch.Tensor, slot_ids: torch.Tensor,
+                      qo_indptr: torch.Tensor, single_token_mode: bool = False, *,
+                      stream=None) -> torch.Tensor:
+    """Gated delta-rule recurrence over each request's tokens with the fp32 state of slot
+    ``slot_ids[b]`` updated in place; returns ``y`` ``(tokens, hv, dv)`` bf16.
+
+    Drop-in for ``mini_sglang_mlx_kernel.gdn_state_inplace`` (bindings.cpp:56-65,
+    gdn_state.cpp:87-135): same argument order, ``single_token_mode`` (decode: one token per
+    request, ``qo_indptr`` ignored) and error texts (gdn_state.cpp:26-84, 107-126).
+    """
+    op = "gdn_state_inplace"
+    if q.dim() != 3 or k.dim() != 3:
+        _fail(op, "q and k must be 3D")
+    if v.dim() != 3:
+        _fail(op, "v must be 3D")
+    if g.dim() != 2 or beta.dim() != 2:
+        _fail(op, "g and beta must be 2D")
+    if state.dim() != 4:
+        _fail(op, "state must be 4D")
+    if slot_ids.dim() != 1 or slot_ids.dtype != torch.int32:
+        _fail(op, "slot_ids must be int32 1D")
+    if any(t.dtype != torch.bfloat16 for t in (q, k, v, g, beta)):
+        _fail(op, "q/k/v/g/beta must be bfloat16")
+    if state.dtype != torch.float32:
+        _fail(op, "state must be float32")
+    if not (q.shape[0] == k.shape[0] == v.shape[0] == g.shape[0] == beta.shape[0]):
+        _fail(op, "leading dimensions must match")
+    if q.shape[1] != k.shape[1] or q.shape[2] != k.shape[2]:
+        _fail(op, "q and k shapes must match")
+    if v.shape[1] != g.shape[1] or v.shape[1] != beta.shape[1]:
+        _fail(op, "hv dimension mismatch")
+    if state.shape[1] != v.shape[1] or state.shape[2] != v.shape[2] or state.shape[3] != q.shape[2]:
+        _fail(op, "state shape must be (slots, hv, dv, dk)")
+    if v.shape[1] % q.shape[1] != 0:
+        _fail(op, "hv must be a multiple of hk")
+    if q.shape[2] != 128 or v.shape[2] != 128:
+        _fail(op, "this specialized kernel requires dk=dv=128")
+    tokens, hk, dk = q.shape
+    hv, dv = v.shape[1], v.shape[2]
+    batch = slot_ids.shape[0]
+    if single_token_mode:
+        if tokens != batch:
+            _fail(op, "decode mode expects one token per request")
+    else:
+        if qo_indptr.dim() != 1 or qo_indptr.dtype != torch.int32:
+            _fail(op, "qo_indptr must be int32 1D")
+        if qo_indptr.shape[0] != batch + 1:
+            _fail(op, "qo_indptr must have shape (batch + 1,)")
+    dev = _require_device(op, q, k, v, g, beta, state, slot_ids)
+    if not single_token_mode and qo_indptr.device != dev:
+        _fail(op, "all tensors must be on the same device")
+    qs, ks, vs = (_heads_stride0(op, t, n) for t, n in ((q, "q"), (k, "k"), (v, "v")))
+    if not (state.stride(3) == 1 and state.stride(2) == dk and state.stride(1) == dv * dk):
+        _fail(op, "state must be contiguous in its (hv, dv, dk) dimensions")
+    state_stride0 = state.stride(0) if state.shape[0] > 1 else hv * dv * dk
+    g, beta = g.contiguous(), beta.contiguous()
+    slot_ids = slot_ids.contiguous()
+    y = torch.empty((tokens, hv, dv), dtype=q.dtype, device=dev)
+    rc = _lib.load().msgl_gdn_state_inplace(
+        q.data_ptr(), k.data_ptr(), v.data_ptr(), g.data_ptr(), beta.data_ptr(), state.data_ptr(),
+        slot_ids.data_ptr(), None if single_token_mode else qo_indptr.contiguous().data_ptr(),
+        y.data_ptr(), tokens, batch, hk, hv, dk, dv, state.shape[0], state_stride0, qs, ks, vs,
+        1 if single_token_mode else 0, _stream_ptr(stream, dev))
+    _check_rc(op, rc)
+    return y

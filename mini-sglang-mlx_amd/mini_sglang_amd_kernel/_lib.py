@@ -44,6 +44,10 @@ SIGNATURES = {
         ctypes.c_int,
         [_vp, _vp, _vp, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64,
          _i64, _i64, _i64, _i64, _f32, _f32, _i32, _vp]),
+    "msgl_gdn_state_inplace": (
+        ctypes.c_int,
+        [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64,
+         _i64, _i64, _i64, _i64, _i32, _vp]),
 }
 
 MSGL_DTYPE_BF16 = 0
@@ -53,6 +57,7 @@ TUNE_MIN_SEGMENT = 1
 TUNE_SMALLQ_MAXCOLS = 2
 TUNE_PREFILL_VARIANT = 3
 TUNE_SPLITKV_WAVES = 4
+TUNE_GDN_ROWS = 5
 
 _lib = None
 
