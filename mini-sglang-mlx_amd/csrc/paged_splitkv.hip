@@ -57,8 +57,7 @@ struct SplitKvParams {
   uint16_t* out;
   float* part_o;        // [n_seg + batch][n_kv][cols][D]
   float* part_lse;      // [n_seg + batch][n_kv][cols]
-  int32_t* req_vstart;  // [batch] stream position of a request's first visible key
-  int32_t* seg_info;    // [0] = segment length the attention kernel used
+  int32_t* req_items;   // [batch][2] first segment holding the request, number of segments sharing it
   int64_t k_stride0, v_stride0;
   int32_t batch, n_q, n_kv, group;
   int32_t nwh;          // kv heads per workgroup
@@ -183,7 +182,6 @@ __global__ __launch_bounds__(64 * NW, ((D == 128 && NCT == 1) ? 2 : 1)) void spl
   const int kvh = (blockIdx.x - seg * p.head_groups) * p.nwh + (wave - cw * p.nwh);
   int seg_len, total, cur_b, vs;
   if (!locate_segment(p, seg, &seg_len, &total, &cur_b, &vs)) return;
-  if (blockIdx.x == 0 && threadIdx.x == 0) p.seg_info[0] = seg_len;
   cur_b = __builtin_amdgcn_readfirstlane(cur_b);
   vs = __builtin_amdgcn_readfirstlane(vs);
   int vpos = seg * seg_len;
@@ -210,7 +208,12 @@ __global__ __launch_bounds__(64 * NW, ((D == 128 && NCT == 1) ? 2 : 1)) void spl
     const int t_begin = r.lo + (vpos - vs);
     const int t_end = min(r.hi, t_begin + (seg_end - vpos));
     const bool whole = (t_begin == r.lo) && (t_end == r.hi);
-    if (t_begin == r.lo && kvh == 0 && ct0 == 0 && lane == 0) p.req_vstart[cur_b] = vs;
+    if (t_begin == r.lo && kvh == 0 && ct0 == 0 && lane == 0) {
+      // the wave that starts a request tells the merge kernel where its partials are
+      const int s_first = vs / seg_len;
+      p.req_items[2 * cur_b] = s_first;
+      p.req_items[2 * cur_b + 1] = (vs + vlen - 1) / seg_len - s_first + 1;
+    }
     const int ncols = r.q_len * p.group;
 
     // ---- Q operand and per-column visibility bounds --------------------------------
@@ -451,28 +454,40 @@ __global__ __launch_bounds__(64) void splitkv_merge_kernel(SplitKvParams p) {
   const int qi = blockIdx.x - b * p.max_len_extend;
   const int hq = blockIdx.y;
   const int lane = lane_id();
+  // two memory round trips in all: the request's geometry and the place of its partials,
+  // then every LSE and the first partial rows together
+  const int s_first = p.req_items[2 * b];
+  const int n_items = p.req_items[2 * b + 1];
   const ReqInfo r = request_info(p, b);
   if (qi >= r.q_len) return;
   constexpr int PER = D / kWave;  // consecutive floats per lane
   uint16_t* orow = p.out + ((int64_t)(r.q_start + qi) * p.n_q + hq) * D + lane * PER;
-  const int vlen = r.hi - r.lo;
-  if (vlen == 0) {
+  if (r.hi - r.lo == 0) {  // no visible key: nobody wrote req_items, the row is zero
 #pragma unroll
     for (int e = 0; e < PER; ++e) orow[e] = 0;
     return;
   }
-  const int seg_len = p.seg_info[0];
-  const int vs = p.req_vstart[b];
-  const int s_first = vs / seg_len;
-  const int n_items = (vs + vlen - 1) / seg_len - s_first + 1;
-  if (n_items == 1) return;
+  if (n_items == 1) return;  // written by the attention kernel itself
   const int kvh = hq / p.group;
   const int col = qi * p.group + (hq - kvh * p.group);
   const int64_t stride = (int64_t)p.n_kv * p.cols;
   const int64_t row0 = ((int64_t)(s_first + b) * p.n_kv + kvh) * p.cols + col;
 
+  constexpr int kAhead = 4;  // partial rows requested before their weights are known
+  float v[kAhead][PER];
+#pragma unroll
+  for (int u = 0; u < kAhead; ++u) {
+    const float* src = p.part_o + (row0 + min(u, n_items - 1) * stride) * D + lane * PER;
+#pragma unroll
+    for (int e = 0; e < PER; ++e) v[u][e] = src[e];
+  }
+  float my_lse = kNegInf;  // lane i holds the LSE of item i (+ 64, + 128, ... folded by max)
   float mx = kNegInf;
-  for (int it = lane; it < n_items; it += kWave) mx = fmaxf(mx, p.part_lse[row0 + it * stride]);
+  for (int it = lane; it < n_items; it += kWave) {
+    const float x = p.part_lse[row0 + it * stride];
+    if (it < kWave) my_lse = x;
+    mx = fmaxf(mx, x);
+  }
 #pragma unroll
   for (int off = 1; off < kWave; off <<= 1) mx = fmaxf(mx, __shfl_xor(mx, off, kWave));
   float acc[PER];
@@ -480,26 +495,16 @@ __global__ __launch_bounds__(64) void splitkv_merge_kernel(SplitKvParams p) {
   for (int e = 0; e < PER; ++e) acc[e] = 0.f;
   float wsum = 0.f;
   if (mx > kNegInf) {
-    int it = 0;
-    for (; it + 4 <= n_items; it += 4) {  // four independent partial rows in flight
-      float w[4], v[4][PER];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int64_t row = row0 + (it + u) * stride;
-        w[u] = p.part_lse[row];
-        const float* src = p.part_o + row * D + lane * PER;
-#pragma unroll
-        for (int e = 0; e < PER; ++e) v[u][e] = src[e];
-      }
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const float wu = fast_exp2(w[u] - mx);
+    for (int u = 0; u < kAhead; ++u) {
+      if (u < n_items) {
+        const float wu = fast_exp2(__shfl(my_lse, u, kWave) - mx);
 #pragma unroll
         for (int e = 0; e < PER; ++e) acc[e] += wu * v[u][e];
         wsum += wu;
       }
     }
-    for (; it < n_items; ++it) {
+    for (int it = kAhead; it < n_items; ++it) {
       const int64_t row = row0 + it * stride;
       const float wu = fast_exp2(p.part_lse[row] - mx);
       const float* src = p.part_o + row * D + lane * PER;
@@ -617,7 +622,7 @@ size_t splitkv_workspace_bytes(int64_t batch, int64_t n_q, int64_t n_kv, int64_t
   const int64_t rows = ((int64_t)n_seg + batch) * n_kv * cols;
   size_t bytes = (size_t)rows * (size_t)head_dim * sizeof(float);  // part_o
   bytes += (size_t)rows * sizeof(float);                           // part_lse
-  bytes += (size_t)(batch + 4) * sizeof(int32_t);                  // req_vstart, seg_info
+  bytes += (size_t)(2 * batch + 4) * sizeof(int32_t);              // req_items
   return (bytes + 255) / 256 * 256 + 256;
 }
 
@@ -645,8 +650,7 @@ int launch_splitkv(const SplitKvArgs& a, hipStream_t stream) {
   char* ws = static_cast<char*>(a.workspace);
   p.part_o = reinterpret_cast<float*>(ws);
   p.part_lse = reinterpret_cast<float*>(ws + (size_t)rows * a.head_dim * sizeof(float));
-  p.req_vstart = reinterpret_cast<int32_t*>(ws + (size_t)rows * (a.head_dim + 1) * sizeof(float));
-  p.seg_info = p.req_vstart + a.batch;
+  p.req_items = reinterpret_cast<int32_t*>(ws + (size_t)rows * (a.head_dim + 1) * sizeof(float));
   p.k_stride0 = a.k_stride0;
   p.v_stride0 = a.v_stride0;
   p.batch = (int32_t)a.batch;
