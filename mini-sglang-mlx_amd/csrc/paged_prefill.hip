@@ -168,14 +168,6 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
     for (int ks = 0; ks < KSTEPS; ++ks) {
       u32x4_t raw = {0u, 0u, 0u, 0u};
       if (valid) raw = ld_global_b128(p.q + off + ks * 16 + h * 8);
-      // q carries the softmax scale (and log2 e) from here on: scores leave the MFMA ready
-      // for exp2, at the price of one more bf16 rounding of q
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const float lo = __builtin_bit_cast(float, raw[e] << 16) * p.scale_log2e;
-        const float hi = __builtin_bit_cast(float, raw[e] & 0xffff0000u) * p.scale_log2e;
-        raw[e] = pack_bf16x2(lo, hi);
-      }
       qreg[rt][ks] = as_bf16x8(raw);
     }
     const int qpos = prefix + qi;
@@ -207,15 +199,10 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
 #pragma unroll
       for (int i = 0; i < 16; ++i) oacc[dt][rt][i] = 0.f;
   float m_run[RT], l_run[RT];
-  // The score MFMAs start from -m (the running row max, 0 while there is none) instead of
-  // from 0, so a half tile's scores arrive already shifted and go straight into exp2.
-  f32x16_t s_init[RT];
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
     m_run[rt] = kNegInf;
     l_run[rt] = 0.f;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) s_init[rt][i] = 0.f;
   }
 
   // ---- moving a tile: wave w owns units w*UPW .. w*UPW+UPW-1; in a unit, lane l fetches
@@ -321,11 +308,15 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
       }
     }
   };
-  // Softmax state of one half tile, decided as soon as its scores exist: alpha = exp2(previous
-  // running max - new one), what O and l must be multiplied by before this half is added.
-  // The scores themselves are left shifted by the new max, ready for exp2.
+  // Softmax state of one half tile, decided as soon as its scores exist:
+  //   mul    factor still to be applied to the scores: the softmax scale on interior halves
+  //          (raw scores; max commutes with a positive scale), 1 on boundary halves, which
+  //          are scaled and masked in place
+  //   m_safe the (lazy) running row max the half's exponentials are taken against
+  //   alpha  exp2(previous max - m_safe): what O and l must be multiplied by first
   struct Stats {
-    float alpha[RT];
+    float mul;
+    float m_safe[RT], alpha[RT];
   };
   auto mask_in_place = [&](Scores& sc, int base) {
 #pragma unroll
@@ -333,7 +324,8 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         const int key = base + 8 * (i >> 2) + 4 * h + (i & 3);
-        if (key < row_lo[rt] || key > row_hi[rt]) sc.s[rt][i] = kNegInf;
+        const float x = sc.s[rt][i] * p.scale_log2e;
+        sc.s[rt][i] = (key < row_lo[rt] || key > row_hi[rt]) ? kNegInf : x;
       }
   };
   auto lane_max = [&](const Scores& sc, float (&mx)[RT]) {
@@ -345,29 +337,18 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
       mx[rt] = m;
     }
   };
-  // mx: per-lane max of scores that are relative to the running max (to 0 if there is none
-  // yet).  The running max only moves when it grows by more than kLazy; then (rarely) the
-  // scores are shifted once more and the MFMA start values are refreshed.
-  auto decide = [&](Scores& sc, const float (&mx)[RT], Stats& st) {
+  auto decide = [&](const float (&mx)[RT], Stats& st) {
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
+      const float m = wave_max_xor(mx[rt] * st.mul, 32);
       const float m_old = m_run[rt];
-      const float ref = (m_old == kNegInf) ? 0.f : m_old;
-      const float cand = ref + wave_max_xor(mx[rt], 32);
-      const float m_new = fmaxf(m_old, cand);
+      const float m_new = fmaxf(m_old, m);
       const float m_use = (m_new - m_old > kLazy) ? m_new : m_old;
-      const float m_safe = (m_use == kNegInf) ? 0.f : m_use;
-      const float shift = m_safe - ref;
-      st.alpha[rt] = fast_exp2(m_old - m_safe);
+      st.m_safe[rt] = (m_use == kNegInf) ? 0.f : m_use;
+      st.alpha[rt] = fast_exp2(m_old - st.m_safe[rt]);
       m_run[rt] = m_use;
+      pin(st.m_safe[rt]);
       pin(st.alpha[rt]);
-      if (__any(shift != 0.f)) {
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          sc.s[rt][i] -= shift;
-          s_init[rt][i] = -m_safe;
-        }
-      }
     }
   };
   // One pipeline step over half tiles i-1, i, i+1.  The matrix pipe computes the scores of
@@ -394,7 +375,7 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
       for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
         for (int i = first; i < first + 8; ++i) {
-          float e = fast_exp2(cur.s[rt][i]);
+          float e = fast_exp2(__builtin_fmaf(cur.s[rt][i], st_cur.mul, -st_cur.m_safe[rt]));
           pin(e);
           cur.s[rt][i] = e;
         }
@@ -419,8 +400,7 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
       for (int e = 0; e < 4; ++e)
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt)
-          nxt.s[rt] = mfma_32x32x16(ops[e], qreg[rt][first + e],
-                                    (first + e == 0) ? s_init[rt] : nxt.s[rt]);
+          nxt.s[rt] = mfma_32x32x16(ops[e], qreg[rt][first + e], nxt.s[rt]);
     };
     auto pv_slice = [&](int u, const bf16x8_t (&ops)[4]) {  // 16 keys, all four dim tiles
 #pragma unroll
@@ -431,7 +411,11 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
     bf16x8_t ops_a[4], ops_b[4];
     // slice 0
 #pragma unroll
-    for (int rt = 0; rt < RT; ++rt) psum[rt] = 0.f;
+    for (int rt = 0; rt < RT; ++rt) {
+      psum[rt] = 0.f;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) nxt.s[rt][i] = 0.f;
+    }
 #pragma unroll
     for (int e = 0; e < 4; ++e) ops_a[e] = k_operand(ks, 4 + e);
     qk_slice(0, kops);
@@ -448,11 +432,13 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
     side(1);
     MSGL_TICK(8 + 4 * prof_half + 1);
     __builtin_amdgcn_sched_barrier(0);
-    if (mask_nxt) {  // boundary half: mask in place
+    st_nxt.mul = p.scale_log2e;
+    if (mask_nxt) {  // boundary half: scale and mask in place
       // the empty volatile statement keeps this a branch: turned into selects it would put
-      // extra VALU instructions into every half tile
+      // 64 extra VALU instructions into every half tile
       asm volatile("" ::: "memory");
       mask_in_place(nxt, nxt_base);
+      st_nxt.mul = 1.0f;
     }
     // slice 2
 #pragma unroll
@@ -472,7 +458,7 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
     pv_slice(1, ops_a);
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) l_run[rt] = l_run[rt] * st_cur.alpha[rt] + psum[rt];
-    decide(nxt, mx, st_nxt);
+    decide(mx, st_nxt);
     side(3);
     MSGL_TICK(8 + 4 * prof_half + 3);
     __builtin_amdgcn_sched_barrier(0);
@@ -484,8 +470,9 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
   // third K and V stages.  Every move is unconditional (tiles past the end clamp to the last
   // key and are fully masked).  A wave waits for its own moves at the end of the iteration,
   // then the workgroup barrier publishes them: one barrier per tile.
+  const bool general_scale = p.scale_log2e <= 0.f;  // fast path needs a positive scale
   auto needs_mask = [&](int base) {  // some row of this wave sees only part of keys base .. base+31
-    return (base < w_lo_max) || (base + 31 > w_hi_min);
+    return general_scale || (base < w_lo_max) || (base + 31 > w_hi_min);
   };
   if (n_tiles > 0) {
     slot_load(k_lo);
@@ -505,15 +492,21 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
     Stats st_a, st_b;
     bf16x8_t pb_a[RT][2], pb_b[RT][2];
     qk_half(0, 0, sa);
-    if (needs_mask(k_lo)) mask_in_place(sa, k_lo);
+    st_a.mul = p.scale_log2e;
+    if (needs_mask(k_lo)) {
+      mask_in_place(sa, k_lo);
+      st_a.mul = 1.0f;
+    }
     {
       float mx[RT];
       lane_max(sa, mx);
-      decide(sa, mx, st_a);
+      decide(mx, st_a);
     }
+    st_b.mul = 1.0f;
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
       st_b.alpha[rt] = 1.0f;
+      st_b.m_safe[rt] = 0.f;
 #pragma unroll
       for (int u = 0; u < 2; ++u) pb_b[rt][u] = as_bf16x8(u32x4_t{0u, 0u, 0u, 0u});
     }

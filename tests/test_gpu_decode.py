@@ -75,3 +75,12 @@ def test_decode_strided_pool_views(gpu):
                                  g.num_kv_splits, g.sm_scale, g.max_kv_splits)
     torch.cuda.synchronize()
     assert_close_bf16(out.cpu(), want, "decode strided pools")
+
+
+@pytest.mark.parametrize("scale", [0.0, -0.3, 1.5])
+def test_decode_unusual_softmax_scales(gpu, scale):
+    import dataclasses
+
+    wl = build_workload("t", "decode", seed=77, n_q=8, n_kv=2, kv_lens=[1, 90, 700, 2100],
+                        pool_factor=1.2)
+    _check(dataclasses.replace(wl, sm_scale=scale), gpu, f"decode scale={scale}")

@@ -119,6 +119,20 @@ def test_head_dim_256_short_and_long_queries(gpu, is_cross, window):
     _check(short, gpu, f"head_dim 256 short cross={is_cross} W={window}")
 
 
+@pytest.mark.parametrize("scale", [0.0, -0.3, 1.5, 0.01])
+def test_unusual_softmax_scales_on_both_routes(gpu, tile_variant, scale):
+    # zero (uniform weights), negative (the smallest score wins), large (peaky rows: the running
+    # max jumps by more than the lazy threshold again and again), tiny
+    import dataclasses
+
+    for extend in ([70, 130, 65], [3, 8, 5]):  # MFMA tile route, split-K route
+        wl = build_workload("t", "prefill", seed=400, n_q=8, n_kv=2,
+                            kv_lens=[70 + extend[0], 300 + extend[1], extend[2]],
+                            extend_lens=extend, pool_factor=1.2, store_new=True)
+        wl = dataclasses.replace(wl, sm_scale=scale)
+        _check(wl, gpu, f"scale={scale} extend={extend} variant={tile_variant}")
+
+
 def test_splitk_route_ragged_q_and_chunking(gpu):
     from mini_sglang_amd_kernel import _lib
 
