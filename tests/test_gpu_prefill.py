@@ -133,6 +133,21 @@ def test_unusual_softmax_scales_on_both_routes(gpu, tile_variant, scale):
         _check(wl, gpu, f"scale={scale} extend={extend} variant={tile_variant}")
 
 
+def test_large_magnitude_inputs_do_not_overflow(gpu, tile_variant):
+    # q and k eight times larger: scores of several hundred (base-2 exponents far beyond what
+    # fp32 exp2 can take without the running max), one key dominating most rows
+    import dataclasses
+
+    for extend in ([70, 130, 65], [3, 8, 5]):
+        wl = build_workload("t", "prefill", seed=410, n_q=8, n_kv=2,
+                            kv_lens=[70 + extend[0], 300 + extend[1], extend[2]],
+                            extend_lens=extend, pool_factor=1.2, store_new=True)
+        wl = dataclasses.replace(wl, q=(wl.q.float() * 8).to(torch.bfloat16),
+                                 k_cache=(wl.k_cache.float() * 8).to(torch.bfloat16),
+                                 new_k=(wl.new_k.float() * 8).to(torch.bfloat16))
+        got = _check(wl, gpu, f"large magnitude extend={extend} variant={tile_variant}")
+
+
 def test_splitk_route_ragged_q_and_chunking(gpu):
     from mini_sglang_amd_kernel import _lib
 
