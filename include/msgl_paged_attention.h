@@ -134,7 +134,8 @@ MSGL_API size_t msgl_paged_prefill_workspace_bytes(int64_t batch, int64_t total_
  * for their first max_len_extend queries, as in the reference's grid
  * (paged_prefill_attention.cpp:152-159).  Short query blocks (speculative verify,
  * draft proposal) are routed to the bandwidth-bound split-K kernel, long ones to
- * the MFMA tile kernel; same arguments, same result.
+ * the MFMA tile kernel (head_dim 128) or, at head_dim 256, to the split-K kernel run
+ * once per chunk of queries; same arguments, same result.
  */
 MSGL_API int msgl_paged_prefill_attention(const void* q, const void* k_cache, const void* v_cache,
                                  const int32_t* qo_indptr, const int32_t* kv_indptr,
