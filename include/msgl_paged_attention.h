@@ -40,7 +40,8 @@
 extern "C" {
 #endif
 
-/* element types of q / k / v / pools / out */
+/* element types of q / k / v / pools / out (F16: store and decode; prefill is bf16 only,
+ * as paged_prefill_attention.metal:646-647) */
 #define MSGL_DTYPE_BF16 0
 #define MSGL_DTYPE_F16 1
 
@@ -104,6 +105,8 @@ MSGL_API size_t msgl_paged_decode_workspace_bytes(int64_t batch, int64_t total_k
  * split hints, backend.py:304-307) are accepted and validated but do not steer
  * the cut.  A request with no tokens gets zeros (the reference leaves its rows
  * unwritten, paged_decode_attention.metal:354).
+ * `dtype`: MSGL_DTYPE_BF16 or MSGL_DTYPE_F16, the two the reference instantiates for decode
+ * (paged_decode_attention.metal:596-604); q, both pools and out share it.
  */
 MSGL_API int msgl_paged_decode_attention(const void* q, const void* k_cache, const void* v_cache,
                                 const int32_t* kv_indptr, const int32_t* kv_indices,

@@ -16,11 +16,13 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 
 int check_common(const void* q, const void* k_cache, const void* v_cache, const void* out,
                  int64_t n_q, int64_t n_kv, int64_t d, int64_t k_stride0, int64_t v_stride0,
-                 int32_t dtype, const char*) {
+                 int32_t dtype, bool f16_ok) {
   if (d != 128 && d != 256) return MSGL_ERR_HEAD_DIM;
   if (n_q <= 0 || n_kv <= 0) return MSGL_ERR_SHAPE;
   if (n_q % n_kv != 0) return MSGL_ERR_HEAD_RATIO;
-  if (dtype != MSGL_DTYPE_BF16) return MSGL_ERR_DTYPE;
+  // IEEE half exists for decode only, as in the reference (paged_decode_attention.metal:596-604
+  // against paged_prefill_attention.metal:646-647)
+  if (dtype != MSGL_DTYPE_BF16 && !(f16_ok && dtype == MSGL_DTYPE_F16)) return MSGL_ERR_DTYPE;
   if (k_stride0 < n_kv * d || v_stride0 < n_kv * d) return MSGL_ERR_SHAPE;
   if (!q || !k_cache || !v_cache || !out) return MSGL_ERR_NULL_POINTER;
   // 16-byte row segments are the unit of every load and store
@@ -130,7 +132,7 @@ int msgl_paged_decode_attention(const void* q, const void* k_cache, const void* 
   if (batch < 0 || total_kv < 0 || num_slots < 0) return MSGL_ERR_SHAPE;
   if (batch == 0) return MSGL_OK;
   int rc = check_common(q, k_cache, v_cache, out, num_q_heads, num_kv_heads, head_dim,
-                        k_cache_stride0, v_cache_stride0, dtype, "paged_decode_attention");
+                        k_cache_stride0, v_cache_stride0, dtype, /*f16_ok=*/true);
   if (rc != MSGL_OK) return rc;
   const int64_t group = num_q_heads / num_kv_heads;
   if (group > 16) return MSGL_ERR_GROUP_TOO_LARGE;  // paged_decode_attention.cpp:54-57
@@ -160,6 +162,7 @@ int msgl_paged_decode_attention(const void* q, const void* k_cache, const void* 
   a.v_stride0 = v_cache_stride0;
   a.sm_scale = sm_scale;
   a.max_len_extend = 1;
+  a.f16 = (dtype == MSGL_DTYPE_F16) ? 1 : 0;
   a.is_cross = 0;
   a.window = 0;
   a.n_seg = n_seg;
@@ -215,7 +218,7 @@ int msgl_paged_prefill_attention(const void* q, const void* k_cache, const void*
   if (total_q < 0 || total_kv < 0 || num_slots < 0) return MSGL_ERR_SHAPE;
   if (total_q == 0 || max_len_extend <= 0) return MSGL_OK;
   int rc = check_common(q, k_cache, v_cache, out, num_q_heads, num_kv_heads, head_dim,
-                        k_cache_stride0, v_cache_stride0, dtype, "paged_prefill_attention");
+                        k_cache_stride0, v_cache_stride0, dtype, /*f16_ok=*/false);
   if (rc != MSGL_OK) return rc;
   if (!qo_indptr || !kv_indptr || !prefix_lens || (total_kv > 0 && !kv_indices))
     return MSGL_ERR_NULL_POINTER;

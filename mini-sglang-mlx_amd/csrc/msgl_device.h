@@ -9,6 +9,8 @@ typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 
@@ -66,6 +68,28 @@ __device__ __forceinline__ f32x4_t mfma_16x16x32(bf16x8_t a, bf16x8_t b, f32x4_t
 //   D: lane l holds D[8*(i/4) + 4*(l/32) + i%4][l%32], i = 0..15
 __device__ __forceinline__ f32x16_t mfma_32x32x16(bf16x8_t a, bf16x8_t b, f32x16_t c) {
   return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+
+// The same product on raw 16-bit operands: bf16 or, with F16, IEEE half.
+template <bool F16>
+__device__ __forceinline__ f32x4_t mfma_16x16x32_raw(u32x4_t a, u32x4_t b, f32x4_t c) {
+  if constexpr (F16)
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, a),
+                                                  __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+  else
+    return mfma_16x16x32(as_bf16x8(a), as_bf16x8(b), c);
+}
+// Two fp32 -> packed 16-bit pair, round to nearest even.
+template <bool F16>
+__device__ __forceinline__ uint32_t pack_16x2(float lo, float hi) {
+  if constexpr (F16) {
+    f16x2_t p;
+    p[0] = (_Float16)lo;
+    p[1] = (_Float16)hi;
+    return __builtin_bit_cast(uint32_t, p);
+  } else {
+    return pack_bf16x2(lo, hi);
+  }
 }
 
 __device__ __forceinline__ float wave_max_xor(float v, int mask) {

@@ -34,6 +34,7 @@ struct SplitKvArgs {
   int32_t max_len_extend;  // 1 for decode; queries per request handled by this launch
   int32_t q_begin;         // first query of every request handled by this launch
   int32_t q_cap;           // cap on a request's query count (0: max_len_extend)
+  int32_t f16;             // 1: q / pools / out are IEEE half (decode only), 0: bf16
   int32_t is_cross, window;
   int32_t n_seg;    // segments the visible token stream is cut into
   int32_t min_seg;  // smallest segment length in tokens, multiple of 64

@@ -64,6 +64,7 @@ struct SplitKvParams {
   int32_t head_groups;  // n_kv / nwh
   int32_t n_seg, min_seg, cols, max_len_extend;
   int32_t q_begin, q_cap;  // first query of every request in this launch; cap on a request's queries
+  int32_t f16;             // elements are IEEE half instead of bf16
   int32_t is_cross, window;
   int32_t wide;  // pool byte offsets need 64 bits
   float scale_log2e;
@@ -167,7 +168,7 @@ struct KvTile {
 // column tile at head dim 128 fits 256 VGPRs, so two such waves per SIMD can be resident.
 // WIDE: pool byte offsets need 64 bits (a pool of 4 GiB or more); otherwise a row's offset is
 // one 32-bit multiply instead of a 64-bit multiply-add per load.
-template <int D, int NCT, int NW, bool WIDE>
+template <int D, int NCT, int NW, bool WIDE, bool F16>
 __global__ __launch_bounds__(64 * NW, ((D == 128 && NCT == 1) ? 2 : 1)) void splitkv_attention_kernel(SplitKvParams p) {
   constexpr int KS = D / 32;   // k-steps of the QK product
   constexpr int VH = D / 128;  // 128-wide halves of D in the PV product
@@ -217,7 +218,7 @@ __global__ __launch_bounds__(64 * NW, ((D == 128 && NCT == 1) ? 2 : 1)) void spl
     const int ncols = r.q_len * p.group;
 
     // ---- Q operand and per-column visibility bounds --------------------------------
-    bf16x8_t qreg[NCT][KS];
+    u32x4_t qreg[NCT][KS];
     int col_lo[NCT], col_hi[NCT];
     int all_lo = 0, all_hi = 0x7fffffff;  // tile is mask-free iff inside [all_lo, all_hi]
 #pragma unroll
@@ -232,7 +233,7 @@ __global__ __launch_bounds__(64 * NW, ((D == 128 && NCT == 1) ? 2 : 1)) void spl
       for (int c = 0; c < KS; ++c) {
         u32x4_t raw = {0u, 0u, 0u, 0u};
         if (valid) raw = ld_global_b128(qrow + c * 32);
-        qreg[ct][c] = as_bf16x8(raw);
+        qreg[ct][c] = raw;
       }
       const int qpos = r.prefix + qi;
       int lo = (p.window > 0) ? qpos - p.window + 1 : 0;
@@ -305,7 +306,7 @@ __global__ __launch_bounds__(64 * NW, ((D == 128 && NCT == 1) ? 2 : 1)) void spl
           f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
           for (int c = 0; c < KS; ++c)
-            acc = mfma_16x16x32(as_bf16x8(t.k[sub][c]), qreg[ct][c], acc);
+            acc = mfma_16x16x32_raw<F16>(t.k[sub][c], qreg[ct][c], acc);
           s[sub][ct] = acc;
         }
       const bool need_mask = (tb < all_lo) || (tb + 31 > all_hi);
@@ -343,10 +344,10 @@ __global__ __launch_bounds__(64 * NW, ((D == 128 && NCT == 1) ? 2 : 1)) void spl
             psum += x[sub][i];
           }
         l_run[ct] = l_run[ct] * alpha + psum;
-        pb[ct][0] = pack_bf16x2(x[0][0], x[0][1]);
-        pb[ct][1] = pack_bf16x2(x[0][2], x[0][3]);
-        pb[ct][2] = pack_bf16x2(x[1][0], x[1][1]);
-        pb[ct][3] = pack_bf16x2(x[1][2], x[1][3]);
+        pb[ct][0] = pack_16x2<F16>(x[0][0], x[0][1]);
+        pb[ct][1] = pack_16x2<F16>(x[0][2], x[0][3]);
+        pb[ct][2] = pack_16x2<F16>(x[1][0], x[1][1]);
+        pb[ct][3] = pack_16x2<F16>(x[1][2], x[1][3]);
         if (__any(alpha != 1.0f)) {
 #pragma unroll
           for (int hf = 0; hf < VH; ++hf)
@@ -369,7 +370,7 @@ __global__ __launch_bounds__(64 * NW, ((D == 128 && NCT == 1) ? 2 : 1)) void spl
 #pragma unroll
           for (int ct = 0; ct < NCT; ++ct) {
             const u32x4_t pv = {pb[ct][0], pb[ct][1], pb[ct][2], pb[ct][3]};
-            oacc[ct][hf][n] = mfma_16x16x32(as_bf16x8(vt), as_bf16x8(pv), oacc[ct][hf][n]);
+            oacc[ct][hf][n] = mfma_16x16x32_raw<F16>(vt, pv, oacc[ct][hf][n]);
           }
         }
     };
@@ -415,7 +416,7 @@ __global__ __launch_bounds__(64 * NW, ((D == 128 && NCT == 1) ? 2 : 1)) void spl
             u32x4_t w;
 #pragma unroll
             for (int n = 0; n < 4; ++n)
-              w[n] = pack_bf16x2(oacc[ct][hf][2 * n][i] * inv, oacc[ct][hf][2 * n + 1][i] * inv);
+              w[n] = pack_16x2<F16>(oacc[ct][hf][2 * n][i] * inv, oacc[ct][hf][2 * n + 1][i] * inv);
             st_global_b128(orow + hf * 128 + (4 * g + i) * 8, w);
           }
       } else {
@@ -448,7 +449,7 @@ __global__ __launch_bounds__(64 * NW, ((D == 128 && NCT == 1) ? 2 : 1)) void spl
 // One wave per (request, query, q head): merge the partials of the segments that share
 // the request, by base-2 LSE.  Requests without visible keys get zeros; requests that sat
 // inside one segment were written by the attention kernel itself.
-template <int D>
+template <int D, bool F16>
 __global__ __launch_bounds__(64) void splitkv_merge_kernel(SplitKvParams p) {
   const int b = blockIdx.x / p.max_len_extend;
   const int qi = blockIdx.x - b * p.max_len_extend;
@@ -516,7 +517,7 @@ __global__ __launch_bounds__(64) void splitkv_merge_kernel(SplitKvParams p) {
   const float inv = (wsum > 0.f) ? 1.0f / wsum : 0.f;
 #pragma unroll
   for (int e = 0; e < PER; e += 2)
-    *reinterpret_cast<uint32_t*>(orow + e) = pack_bf16x2(acc[e] * inv, acc[e + 1] * inv);
+    *reinterpret_cast<uint32_t*>(orow + e) = pack_16x2<F16>(acc[e] * inv, acc[e + 1] * inv);
 }
 
 int nct_for(int64_t cols) { return (int)((cols + 15) / 16); }
@@ -547,12 +548,20 @@ int device_cus() {
 template <int D, int NCT, int NW>
 void launch_attn(const SplitKvParams& p, hipStream_t stream) {
   const dim3 grid((unsigned)(p.n_seg * p.head_groups)), block(64 * NW);
-  if (p.wide) hipLaunchKernelGGL((splitkv_attention_kernel<D, NCT, NW, true>), grid, block, 0, stream, p);
-  else hipLaunchKernelGGL((splitkv_attention_kernel<D, NCT, NW, false>), grid, block, 0, stream, p);
+  if constexpr (NCT == 1) {  // IEEE half exists for decode only (one column tile)
+    if (p.f16) {
+      if (p.wide) hipLaunchKernelGGL((splitkv_attention_kernel<D, NCT, NW, true, true>), grid, block, 0, stream, p);
+      else hipLaunchKernelGGL((splitkv_attention_kernel<D, NCT, NW, false, true>), grid, block, 0, stream, p);
+      return;
+    }
+  }
+  if (p.wide) hipLaunchKernelGGL((splitkv_attention_kernel<D, NCT, NW, true, false>), grid, block, 0, stream, p);
+  else hipLaunchKernelGGL((splitkv_attention_kernel<D, NCT, NW, false, false>), grid, block, 0, stream, p);
 }
 
 template <int D, int NCT>
 int launch_dn(const SplitKvParams& p, int waves, hipStream_t stream) {
+  if (p.f16 && NCT != 1) return MSGL_ERR_DTYPE;
   switch (waves) {
     case 1: launch_attn<D, NCT, 1>(p, stream); break;
     case 2: launch_attn<D, NCT, 2>(p, stream); break;
@@ -566,7 +575,8 @@ int launch_dn(const SplitKvParams& p, int waves, hipStream_t stream) {
   int rc = check_launch();
   if (rc != MSGL_OK) return rc;
   const dim3 mgrid((unsigned)(p.batch * p.max_len_extend), (unsigned)p.n_q);
-  hipLaunchKernelGGL((splitkv_merge_kernel<D>), mgrid, dim3(64), 0, stream, p);
+  if (p.f16) hipLaunchKernelGGL((splitkv_merge_kernel<D, true>), mgrid, dim3(64), 0, stream, p);
+  else hipLaunchKernelGGL((splitkv_merge_kernel<D, false>), mgrid, dim3(64), 0, stream, p);
   return check_launch();
 }
 
@@ -662,6 +672,7 @@ int launch_splitkv(const SplitKvArgs& a, hipStream_t stream) {
   p.n_seg = a.n_seg;
   p.min_seg = a.min_seg;
   p.max_len_extend = a.max_len_extend;
+  p.f16 = a.f16;
   p.q_begin = a.q_begin;
   p.q_cap = a.q_cap > 0 ? a.q_cap : a.max_len_extend;
   p.is_cross = a.is_cross;

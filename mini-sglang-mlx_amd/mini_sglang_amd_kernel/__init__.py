@@ -114,15 +114,16 @@ def store_kv_cache(k_cache: torch.Tensor, v_cache: torch.Tensor, indices: torch.
     _check_rc(op, rc)
 
 
-def _attention_dtype(op: str, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor) -> int:
+def _attention_dtype(op: str, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                     half_ok: bool) -> int:
     if q.dtype not in _DTYPE_CODE:
         _fail(op, "unsupported dtype, must be float16 or bfloat16")
     if k_cache.dtype != q.dtype or v_cache.dtype != q.dtype:
         _fail(op, "q, k_cache and v_cache must have the same dtype")
-    if q.dtype != torch.bfloat16:
-        # the reference ships no float16 prefill kernel either
-        # (paged_prefill_attention.metal:646-647); this build is bfloat16 throughout
-        _fail(op, "unsupported dtype, this build provides bfloat16 kernels only")
+    if q.dtype != torch.bfloat16 and not half_ok:
+        # float16 exists for decode only, as in the reference: its prefill kernel is
+        # instantiated for bfloat16 alone (paged_prefill_attention.metal:646-647)
+        _fail(op, "unsupported dtype, the prefill kernel is bfloat16 only")
     return _DTYPE_CODE[q.dtype]
 
 
@@ -165,7 +166,7 @@ def paged_decode_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torc
         _fail(op, "cache head_dim must match q head_dim")
     if v_cache.shape[1] != num_kv_heads:
         _fail(op, "v_cache shape must match k_cache")
-    dtype = _attention_dtype(op, q, k_cache, v_cache)
+    dtype = _attention_dtype(op, q, k_cache, v_cache, half_ok=True)
     kv_indptr = _int32_1d(op, kv_indptr, "kv_indptr")
     kv_indices = _int32_1d(op, kv_indices, "kv_indices")
     num_kv_splits = _int32_1d(op, num_kv_splits, "num_kv_splits")
@@ -233,7 +234,7 @@ def paged_prefill_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
         _fail(op, "batch must be > 0")
     if v_cache.shape[1] != num_kv_heads:
         _fail(op, "v_cache shape must match k_cache")
-    dtype = _attention_dtype(op, q, k_cache, v_cache)
+    dtype = _attention_dtype(op, q, k_cache, v_cache, half_ok=False)
     qo_indptr = _int32_1d(op, qo_indptr, "qo_indptr")
     kv_indptr = _int32_1d(op, kv_indptr, "kv_indptr")
     kv_indices = _int32_1d(op, kv_indices, "kv_indices")

@@ -58,19 +58,20 @@ def test_c_abi_argument_checks_return_codes_without_touching_a_gpu():
     assert dec(d=64) == -2
     assert dec(n_q=30) == -3
     assert dec(n_q=34, n_kv=2) == -4
-    assert dec(dtype=1) == -5
+    assert dec(dtype=2) == -5
     assert dec(q=None) == -1
     assert dec(ws=None) == -8
     assert dec(ws_bytes=16) == -8
     # prefill: window, batch
-    def pre(batch=2, window=0, d=128, n_q=32):
+    def pre(batch=2, window=0, d=128, n_q=32, dtype=0):
         return lib.msgl_paged_prefill_attention(fake, fake, fake, fake, fake, fake, fake, fake,
                                                 fake, 1 << 40, batch, 16, 100, n_q, 8, d, 64,
-                                                8 * d, 8 * d, 0.1, 8, 0, window, 0, None)
+                                                8 * d, 8 * d, 0.1, 8, 0, window, dtype, None)
     assert pre(window=-1) == -7
     assert pre(batch=0) == -6
     assert pre(d=96) == -2
     assert pre(n_q=33) == -3
+    assert pre(dtype=1) == -5  # float16 exists for decode only
     assert lib.msgl_set_tuning(99, 1) == -9
     assert lib.msgl_paged_decode_workspace_bytes(4, 1000, 32, 8, 128) > 0
     assert lib.msgl_paged_decode_workspace_bytes(4, 1000, 30, 8, 128) == 0
