@@ -137,8 +137,7 @@ MSGL_API size_t msgl_paged_prefill_workspace_bytes(int64_t batch, int64_t total_
  * for their first max_len_extend queries, as in the reference's grid
  * (paged_prefill_attention.cpp:152-159).  Short query blocks (speculative verify,
  * draft proposal) are routed to the bandwidth-bound split-K kernel, long ones to
- * the MFMA tile kernel (head_dim 128) or, at head_dim 256, to the split-K kernel run
- * once per chunk of queries; same arguments, same result.
+ * the MFMA tile kernel of their head_dim; same arguments, same result.
  */
 MSGL_API int msgl_paged_prefill_attention(const void* q, const void* k_cache, const void* v_cache,
                                  const int32_t* qo_indptr, const int32_t* kv_indptr,
@@ -232,7 +231,8 @@ MSGL_API int msgl_gdn_state_inplace(const void* q, const void* k, const void* v,
  *   MSGL_TUNE_SEGMENTS       segments the split-K kernel cuts the visible token stream into
  *   MSGL_TUNE_MIN_SEGMENT    smallest segment length in tokens (multiple of 64)
  *   MSGL_TUNE_SMALLQ_MAXCOLS largest q_len*group routed to the split-K kernel
- *   MSGL_TUNE_PREFILL_VARIANT tiling of the MFMA kernel (0: 8 waves x 32 rows, 1: 4 x 64)
+ *   MSGL_TUNE_PREFILL_VARIANT tiling of the head_dim 128 MFMA kernel (0: 8 waves x 32 rows,
+ *                            1: 4 x 64); 2: head_dim 256 through split-K in query chunks
  *   MSGL_TUNE_SPLITKV_WAVES  most waves (adjacent kv heads) per split-K workgroup: 1, 2, 4, 8
  *                            (0 restores the default, 4)
  *   MSGL_TUNE_GDN_ROWS       state rows per 16-lane group of the gdn_state kernel: 1, 2, 4

@@ -20,7 +20,7 @@ LIB_PATH = os.path.join(LIB_DIR, "libmsgl_paged_attention.so")
 # benchmarking aid (measured MFMA ceiling under the board's power limit); bench.py loads it
 PROBE_SRC = os.path.join(CSRC, "probes", "mfma_rate_probe.hip")
 PROBE_PATH = os.path.join(LIB_DIR, "libmsgl_probes.so")
-SOURCES = ["api.hip", "store_kv_cache.hip", "paged_splitkv.hip", "paged_prefill.hip",
+SOURCES = ["api.hip", "store_kv_cache.hip", "paged_splitkv.hip", "paged_prefill.hip", "paged_prefill_d256.hip",
            "build_metadata.hip", "qk_norm_rope_store.hip",
            "gdn_state.hip"]
 

@@ -173,10 +173,11 @@ int msgl_paged_decode_attention(const void* q, const void* k_cache, const void* 
 static bool use_splitkv_route(int64_t group, int64_t max_len_extend) {
   return max_len_extend >= 1 && group * max_len_extend <= smallq_max_cols();
 }
-// The MFMA tile kernel exists for head_dim 128.  Longer queries at head_dim 256 run the
-// split-K kernel once per chunk of queries (each launch re-reads the visible keys).
+// Longer queries run the MFMA tile kernels.  The older route for head_dim 256, the split-K
+// kernel once per chunk of queries (each launch re-reads the visible keys), is kept behind
+// MSGL_TUNE_PREFILL_VARIANT = 2 for comparison.
 static bool use_chunked_route(int64_t head_dim, int64_t group) {
-  return head_dim != 128 && group <= msgl::kSplitKvMaxCols;
+  return head_dim == 256 && msgl::tile_variant() == 2 && group <= msgl::kSplitKvMaxCols;
 }
 static int32_t chunk_queries(int64_t group) {
   return (int32_t)std::max<int64_t>(1, std::min<int64_t>(smallq_max_cols(), msgl::kSplitKvMaxCols) / group);
@@ -286,7 +287,7 @@ int msgl_paged_prefill_attention(const void* q, const void* k_cache, const void*
   a.max_len_extend = max_len_extend;
   a.is_cross = is_cross_attention ? 1 : 0;
   a.window = sliding_window_size;
-  return msgl::launch_prefill_tile(a, s);
+  return head_dim == 256 ? msgl::launch_prefill_tile256(a, s) : msgl::launch_prefill_tile(a, s);
 }
 
 int msgl_build_attention_metadata(const int32_t* page_table, int64_t table_stride0,

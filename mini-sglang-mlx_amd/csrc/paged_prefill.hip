@@ -31,6 +31,7 @@
 #include "msgl_device.h"
 #include "msgl_internal.h"
 #include "prefill_params.h"
+#include "prefill_tile_common.h"
 
 namespace msgl {
 namespace {
@@ -43,10 +44,6 @@ namespace {
 #define MSGL_PROF_HALF(x) do { } while (0)
 #endif
 
-typedef short s16x4_t __attribute__((ext_vector_type(4)));
-constexpr bf16x2_t kOnes = {(__bf16)1.0f, (__bf16)1.0f};
-#define MSGL_LDS_PTR(T, p) ((__attribute__((address_space(3))) T*)(p))
-
 constexpr int kUnitRows = 4;                 // rows moved by one LDS-direct load
 constexpr int kUnits = kBN / kUnitRows;      // 16 per tile
 constexpr int kKUnit = 1024 + 16;            // bytes between K units
@@ -56,37 +53,6 @@ constexpr int kVStage = kUnits * kVUnit;     // 17408
 constexpr int kKStages = 3, kVStages = 3;
 constexpr int kVBase = kKStages * kKStage;
 constexpr int kStageTotal = kVBase + kVStages * kVStage;
-
-// 64 lanes x 16 bytes: lane l's 16 bytes at `saddr + voff` land at LDS byte lds_addr + 16 l.
-// The compiler does not see the LDS write: callers wait on vmcnt and pass a barrier before
-// anyone reads the destination.  M0 is written without telling the compiler (it cannot be
-// named as a clobber); nothing else in these kernels uses M0.
-__device__ __forceinline__ void lds_direct_b128(uint32_t lds_addr, const void* saddr, uint32_t voff) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-               :
-               : "s"(lds_addr), "v"(voff), "s"(saddr)
-               : "memory");
-}
-__device__ __forceinline__ void lds_direct_b128(uint32_t lds_addr, const void* saddr, uint64_t voff) {
-  const unsigned char* a = static_cast<const unsigned char*>(saddr) + voff;
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
-               :
-               : "s"(lds_addr), "v"(a)
-               : "memory");
-}
-// s_waitcnt vmcnt(0) (expcnt and lgkmcnt fields left at their maxima).  Issued through the
-// builtin so that the compiler's own wait bookkeeping sees it.
-__device__ __forceinline__ void wait_all_vm() {
-  __builtin_amdgcn_s_waitcnt(0x0F70);
-  asm volatile("" ::: "memory");
-}
-
-// Lane i of each 16-lane group receives element (i % 4) of the 8 bytes addressed by lanes
-// i/4, 4 + i/4, 8 + i/4, 12 + i/4 of its group.
-__device__ __forceinline__ u32x2_t lds_read_tr16(const unsigned char* p) {
-  const s16x4_t v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(MSGL_LDS_PTR(s16x4_t, p));
-  return __builtin_bit_cast(u32x2_t, v);
-}
 
 // RT = 32-row tiles per wave, NW = waves per workgroup; the workgroup covers NW*RT*32 rows.
 // WIDE: pool byte offsets need 64 bits (pool of 4 GiB or more).

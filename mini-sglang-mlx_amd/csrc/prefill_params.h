@@ -27,11 +27,13 @@ constexpr int kBN = 64;  // keys per tile
 // A stale row max is kept until the new one exceeds it by this much (base-2 exponent):
 // P stays below 2^kLazy, far inside bf16 / fp32 range, and O is rescaled rarely.
 constexpr float kLazy = 8.0f;
-constexpr int kPrefillBlockRows = 256;
+constexpr int kPrefillBlockRows = 256;      // rows per workgroup, head_dim 128
+constexpr int kPrefillBlockRows256 = 128;   // head_dim 256
 
 // Fills `p` and the grid size; returns MSGL_OK, or an error, or sets n_blocks = 0 for an
 // empty problem.  wide: some pool byte offset needs more than 32 bits.
-inline int make_prefill_params(const PrefillArgs& a, PrefillParams& p, int64_t& n_blocks, bool& wide) {
+inline int make_prefill_params(const PrefillArgs& a, PrefillParams& p, int64_t& n_blocks, bool& wide,
+                               int block_rows = kPrefillBlockRows) {
   p.q = static_cast<const uint16_t*>(a.q);
   p.k_cache = static_cast<const uint16_t*>(a.k_cache);
   p.v_cache = static_cast<const uint16_t*>(a.v_cache);
@@ -51,7 +53,7 @@ inline int make_prefill_params(const PrefillArgs& a, PrefillParams& p, int64_t& 
   p.window = a.window;
   p.scale_log2e = a.sm_scale * 1.4426950408889634f;
   const int64_t rows = (int64_t)a.max_len_extend * p.group;
-  const int64_t n_qblk = (rows + kPrefillBlockRows - 1) / kPrefillBlockRows;
+  const int64_t n_qblk = (rows + block_rows - 1) / block_rows;
   const int64_t n_pairs = a.batch * a.n_kv;
   n_blocks = (n_pairs + 7) / 8 * 8 * n_qblk;
   if (n_qblk <= 0 || n_blocks <= 0) {

@@ -1,0 +1,51 @@
+// LDS-direct loads, counted waits and transposing LDS reads shared by the prefill tile kernels.
+#pragma once
+#include "msgl_device.h"
+
+namespace msgl {
+
+typedef short s16x4_t __attribute__((ext_vector_type(4)));
+constexpr bf16x2_t kOnes = {(__bf16)1.0f, (__bf16)1.0f};
+#define MSGL_LDS_PTR(T, p) ((__attribute__((address_space(3))) T*)(p))
+
+// 64 lanes x 16 bytes: lane l's 16 bytes at `saddr + voff` land at LDS byte lds_addr + 16 l.
+// The compiler does not see the LDS write: callers wait on vmcnt and pass a barrier before
+// anyone reads the destination.  M0 is written without telling the compiler (it cannot be
+// named as a clobber); nothing else in these kernels uses M0.
+__device__ __forceinline__ void lds_direct_b128(uint32_t lds_addr, const void* saddr, uint32_t voff) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(lds_addr), "v"(voff), "s"(saddr)
+               : "memory");
+}
+__device__ __forceinline__ void lds_direct_b128(uint32_t lds_addr, const void* saddr, uint64_t voff) {
+  const unsigned char* a = static_cast<const unsigned char*>(saddr) + voff;
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+               :
+               : "s"(lds_addr), "v"(a)
+               : "memory");
+}
+// s_waitcnt vmcnt(0) (expcnt and lgkmcnt fields left at their maxima).  Issued through the
+// builtin so that the compiler's own wait bookkeeping sees it.
+__device__ __forceinline__ void wait_all_vm() {
+  __builtin_amdgcn_s_waitcnt(0x0F70);
+  asm volatile("" ::: "memory");
+}
+
+// s_waitcnt vmcnt(N): returns once at most N of this wave's vector-memory loads are still in
+// flight.  Loads complete in issue order, so this waits for everything older than the last N.
+template <int N>
+__device__ __forceinline__ void wait_vm_at_most() {
+  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit field");
+  __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
+  asm volatile("" ::: "memory");
+}
+
+// Lane i of each 16-lane group receives element (i % 4) of the 8 bytes addressed by lanes
+// i/4, 4 + i/4, 8 + i/4, 12 + i/4 of its group.
+__device__ __forceinline__ u32x2_t lds_read_tr16(const unsigned char* p) {
+  const s16x4_t v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(MSGL_LDS_PTR(s16x4_t, p));
+  return __builtin_bit_cast(u32x2_t, v);
+}
+
+}  // namespace msgl

@@ -101,22 +101,92 @@ def test_splitk_route_masks(gpu, q_len, is_cross, window):
     _check(wl, gpu, f"split-K route q_len={q_len} cross={is_cross} W={window}")
 
 
+@pytest.fixture(params=[0, 2], ids=["tile256", "chunked-splitk"])
+def d256_route(request):
+    """head_dim 256 extends run the 256-wide MFMA tile kernel; the older route (the split-K
+    kernel once per chunk of queries) stays selectable and is checked too."""
+    from mini_sglang_amd_kernel import _lib
+
+    _lib.set_tuning(_lib.TUNE_PREFILL_VARIANT, request.param)
+    yield request.param
+    _lib.set_tuning(_lib.TUNE_PREFILL_VARIANT, 0)
+
+
 @pytest.mark.parametrize("is_cross,window", MASKS)
-def test_head_dim_256_short_and_long_queries(gpu, is_cross, window):
-    # head_dim 256 has no MFMA tile kernel: short query blocks take the split-K route in one
-    # launch, longer ones run it once per chunk of queries (here 64 / group = 16 per launch;
-    # extends of 5, 16, 40 and 70 give a request that ends inside the first chunk, one that
-    # fills it exactly, and two that span three and five chunks)
+def test_head_dim_256_short_and_long_queries(gpu, d256_route, is_cross, window):
+    # extends of 5, 16, 40 and 70 at group 4: the first two are short query blocks (split-K
+    # route in one launch), the others go to the tile kernel (or, chunked, span three and five
+    # launches of 16 queries)
     wl = build_workload("t", "prefill", seed=330, n_q=8, n_kv=2, head_dim=256,
                         kv_lens=[5, 100 + 16, 300 + 40, 70], extend_lens=[5, 16, 40, 70],
                         pool_factor=1.2, store_new=True,
                         is_cross_attention=is_cross, sliding_window_size=window)
-    _check(wl, gpu, f"head_dim 256 chunked cross={is_cross} W={window}")
+    _check(wl, gpu, f"head_dim 256 route={d256_route} cross={is_cross} W={window}")
     short = build_workload("t", "prefill", seed=331, n_q=8, n_kv=2, head_dim=256,
                            kv_lens=[7, 200 + 7, 64 + 3], extend_lens=[7, 7, 3], pool_factor=1.2,
                            store_new=True, is_cross_attention=is_cross,
                            sliding_window_size=window)
     _check(short, gpu, f"head_dim 256 short cross={is_cross} W={window}")
+
+
+@pytest.mark.parametrize("is_cross,window", MASKS)
+def test_head_dim_256_tile_kernel_masks(gpu, is_cross, window):
+    # ragged extends with and without prefix: lengths around the 32-key step (31, 32, 33, 65),
+    # an odd and an even number of steps, several q blocks of 128 rows per (request, kv head)
+    wl = build_workload("t", "prefill", seed=340, n_q=8, n_kv=2, head_dim=256,
+                        kv_lens=[70, 300, 64 + 130, 33, 513 + 65, 31, 32, 1000 + 97],
+                        extend_lens=[70, 100, 130, 33, 65, 31, 32, 97], pool_factor=1.3,
+                        store_new=True, is_cross_attention=is_cross, sliding_window_size=window)
+    _check(wl, gpu, f"head_dim 256 tile kernel cross={is_cross} W={window}")
+
+
+@pytest.mark.parametrize("n_q,n_kv", [(8, 8), (32, 8), (12, 4), (16, 1), (24, 1)])
+def test_head_dim_256_tile_kernel_group_sizes(gpu, n_q, n_kv):
+    wl = build_workload("t", "prefill", seed=350 + n_q, n_q=n_q, n_kv=n_kv, head_dim=256,
+                        kv_lens=[200 + 96, 129, 1000 + 257, 2100 + 70], extend_lens=[96, 129, 257, 70],
+                        pool_factor=1.2, store_new=True)
+    _check(wl, gpu, f"head_dim 256 tile kernel n_q={n_q} n_kv={n_kv}")
+
+
+def test_head_dim_256_tile_kernel_long_prefix_and_chunked_extend(gpu):
+    """A long cached prefix (hundreds of pipeline steps through the stage rings), and one
+    extend computed in two chunks against the same extend in one piece."""
+    import dataclasses
+
+    wl = build_workload("t", "prefill", seed=360, n_q=8, n_kv=2, head_dim=256,
+                        kv_lens=[9000 + 300, 4097 + 200], extend_lens=[300, 200],
+                        pool_factor=1.1, store_new=True)
+    print("head_dim 256 long prefix", flush=True)
+    got, g = run_gpu(wl, gpu)
+    want, _ = run_oracle(wl)
+    assert_close_bf16(got, want, "head_dim 256 long prefix")
+    # the second 150 queries of request 0 as an extend of their own on top of prefix + 150
+    from mini_sglang_amd_kernel import paged_prefill_attention
+    from _util import indptr
+
+    kv0 = 9000 + 300
+    rows = slice(150, 300)
+    out = paged_prefill_attention(
+        g.q[rows], g.k_cache, g.v_cache, indptr([150]).to(gpu), indptr([kv0]).to(gpu),
+        g.kv_indices[:kv0], torch.tensor([9000 + 150], dtype=torch.int32, device=gpu),
+        wl.sm_scale, 150)
+    torch.cuda.synchronize()
+    assert_close_bf16(out.cpu(), got[rows].float(), "head_dim 256 chunked extend", max_tol=8e-3,
+                      mean_tol=4e-4)
+
+
+@pytest.mark.parametrize("scale", [0.0, -0.3, 1.5])
+def test_head_dim_256_tile_kernel_unusual_scales_and_magnitudes(gpu, scale):
+    import dataclasses
+
+    wl = build_workload("t", "prefill", seed=370, n_q=8, n_kv=2, head_dim=256,
+                        kv_lens=[70 + 70, 300 + 130, 65], extend_lens=[70, 130, 65],
+                        pool_factor=1.2, store_new=True)
+    _check(dataclasses.replace(wl, sm_scale=scale), gpu, f"head_dim 256 scale={scale}")
+    big = dataclasses.replace(wl, q=(wl.q.float() * 6).to(torch.bfloat16),
+                              k_cache=(wl.k_cache.float() * 6).to(torch.bfloat16),
+                              new_k=(wl.new_k.float() * 6).to(torch.bfloat16))
+    _check(big, gpu, "head_dim 256 large magnitude")
 
 
 @pytest.mark.parametrize("scale", [0.0, -0.3, 1.5, 0.01])
