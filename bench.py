@@ -135,7 +135,10 @@ def run_config(cfg: int, variant: str, steps: int, warmup: int, check: bool, cpu
 
     t0 = time.time()
     # multi-GiB pools of the long-context shape are drawn on the GPU; the rest on the host
-    wl = config_workload(cfg, variant=variant, pool_device=dev if cfg == 4 else None)
+    if variant == "head_dim_256":
+        wl = config_workload(cfg, head_dim=256)
+    else:
+        wl = config_workload(cfg, variant=variant, pool_device=dev if cfg == 4 else None)
     g = wl.to(dev)
     gen_s = time.time() - t0
     step = make_step(g)
@@ -400,7 +403,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--configs", default="2,3,1,5,5w,4")
+    ap.add_argument("--configs", default="2,3,1,5,5w,4,3h")
     ap.add_argument("--no-check", action="store_true", help="skip the oracle comparison")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--tune", action="append", default=[], metavar="KNOB=VALUE",
@@ -446,7 +449,9 @@ def main():
 
     rows = []
     for tok in [t.strip() for t in args.configs.split(",") if t.strip()]:
-        cfg, variant = (int(tok[:-1]), "window") if tok.endswith("w") else (int(tok), "")
+        # "5w": shape 5 with the sliding window; "3h": shape 3 at head_dim 256
+        suffix = {"w": "window", "h": "head_dim_256"}.get(tok[-1], "")
+        cfg, variant = (int(tok[:-1]), suffix) if suffix else (int(tok), "")
         steps = args.steps if cfg != 4 else max(5, args.steps // 5)
         budget = 0.0 if args.no_cpu_baseline else args.cpu_flops
         row = run_config(cfg, variant, steps, args.warmup if cfg != 4 else max(2, args.warmup // 3),
@@ -463,7 +468,8 @@ def main():
 
     def find(cfg, variant_window=False):
         for r in rows:
-            if r["config"] == cfg and (r["sliding_window"] > 0) == variant_window:
+            if (r["config"] == cfg and (r["sliding_window"] > 0) == variant_window
+                    and r["head_dim"] == 128):
                 return r
         return None
 

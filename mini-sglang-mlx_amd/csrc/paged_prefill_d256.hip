@@ -42,9 +42,9 @@ constexpr int kKUnit = 1024 + 16;             // bytes between K units
 constexpr int kVUnit = 1024 + 64;             // bytes between V units
 constexpr int kKStage = kUnits * kKUnit;      // 16640
 constexpr int kVStage = kUnits * kVUnit;      // 17408
-constexpr int kKStages = 4, kVStages = 3;
+constexpr int kKStages = 4, kVStages = 4;
 constexpr int kVBase = kKStages * kKStage;
-constexpr int kStageTotal = kVBase + kVStages * kVStage;  // 118784
+constexpr int kStageTotal = kVBase + kVStages * kVStage;  // 136192
 constexpr int kKSteps = kD / 16;              // k-steps of QK^T
 constexpr int kDT = kD / 32;                  // 32-dim tiles of O^T
 constexpr int kMovesPerStep = 2 * kUPW;       // V units then K units, per wave
@@ -161,33 +161,36 @@ __global__ __launch_bounds__(kNW * 64) void prefill_tile256_kernel(PrefillParams
   const uint32_t chunk_off = (uint32_t)(lane & 31) * 16u;
   const bool upper = lane >= 32;
   struct Slots {
-    int32_t s[kUPW][2];  // slot ids of the two keys of each of this wave's units (uniform)
+    int32_t s[2][kUPW];  // slot ids of this wave's keys: [0] keys 4w+i, [1] keys 4w+i+16 (uniform)
   };
+  // slot ids of the half starting at key `base`: two 16-byte scalar loads when the half lies
+  // inside the request, element-wise clamped loads on its last, partial half
   auto slot_load = [&](int base, Slots& sl) {
+    const int first = base + w * kUPW;
+    if (first + 16 + kUPW <= kn) {
 #pragma unroll
-    for (int i = 0; i < kUPW; ++i) {
-      sl.s[i][0] = idx_base[min(base + w * kUPW + i, kn - 1)];
-      sl.s[i][1] = idx_base[min(base + w * kUPW + i + 16, kn - 1)];
+      for (int r = 0; r < 2; ++r)
+#pragma unroll
+        for (int i = 0; i < kUPW; ++i) sl.s[r][i] = idx_base[first + 16 * r + i];
+    } else {
+#pragma unroll
+      for (int r = 0; r < 2; ++r)
+#pragma unroll
+        for (int i = 0; i < kUPW; ++i) sl.s[r][i] = idx_base[min(first + 16 * r + i, kn - 1)];
     }
   };
-  auto lane_offset = [&](const int32_t (&s)[2], uint32_t row_bytes) -> OffT {
-    const OffT a = (OffT)(uint32_t)s[0] * row_bytes;  // uniform: scalar multiplies
-    const OffT c = (OffT)(uint32_t)s[1] * row_bytes;
-    return (upper ? c : a) + chunk_off;
+  auto lane_offset = [&](int32_t s_lo, int32_t s_hi, uint32_t row_bytes) -> OffT {
+    const uint32_t slot = (uint32_t)(upper ? s_hi : s_lo);
+    if constexpr (WIDE) return (uint64_t)slot * row_bytes + chunk_off;
+    else return __umul24(slot, row_bytes) + chunk_off;  // both factors below 2^24 here
   };
-  OffT k_off[kUPW], v_off[kUPW];
-  auto k_offsets = [&](const Slots& sl) {
-#pragma unroll
-    for (int i = 0; i < kUPW; ++i) k_off[i] = lane_offset(sl.s[i], k_row_bytes);
-  };
-  auto v_offsets = [&](const Slots& sl) {
-#pragma unroll
-    for (int i = 0; i < kUPW; ++i) v_off[i] = lane_offset(sl.s[i], v_row_bytes);
-  };
+  // K offsets of the half whose K leaves in this step; V offsets of the halves whose V leaves in
+  // this step (`v_off[par]`, computed two steps ago from the same slot ids as that half's K)
+  OffT k_off[kUPW], v_off[2][kUPW];
   // move number n of a step: the V units first, then the K units
-  auto move = [&](int n, uint32_t k_stage, uint32_t v_stage) {
+  auto move = [&](int n, uint32_t k_stage, uint32_t v_stage, const OffT (&voff)[kUPW]) {
     if (n < kUPW)
-      lds_direct_b128(lds0 + v_stage + (uint32_t)(w * kUPW + n) * kVUnit, v_src, v_off[n]);
+      lds_direct_b128(lds0 + v_stage + (uint32_t)(w * kUPW + n) * kVUnit, v_src, voff[n]);
     else
       lds_direct_b128(lds0 + k_stage + (uint32_t)(w * kUPW + n - kUPW) * kKUnit, k_src, k_off[n - kUPW]);
   };
@@ -211,23 +214,6 @@ __global__ __launch_bounds__(kNW * 64) void prefill_tile256_kernel(PrefillParams
     const u32x2_t hi = lds_read_tr16(vs + u * 512 + dt * 64 + 8 * kVUnit);
     return as_bf16x8(u32x4_t{lo[0], lo[1], hi[0], hi[1]});
   };
-  auto rescale = [&](float alpha) {
-    if (__any(alpha != 1.0f)) {
-#pragma unroll
-      for (int dt = 0; dt < kDT; ++dt)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) oacc[dt][i] *= alpha;
-    }
-  };
-  // Softmax state of one half, decided as soon as its scores exist:
-  //   mul    factor still to be applied to the scores: the softmax scale on interior halves
-  //          (max commutes with a positive scale), 1 on boundary halves, which are scaled and
-  //          masked in place
-  //   m_safe the (lazy) running row max the half's exponentials are taken against
-  //   alpha  exp2(previous max - m_safe): what O and l must be multiplied by first
-  struct Stats {
-    float mul, m_safe, alpha;
-  };
   auto mask_in_place = [&](f32x16_t& s, int base) {
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
@@ -236,38 +222,69 @@ __global__ __launch_bounds__(kNW * 64) void prefill_tile256_kernel(PrefillParams
       s[i] = (key < row_lo || key > row_hi) ? kNegInf : x;
     }
   };
-  auto lane_max = [&](const f32x16_t& s) {
-    float m = fmaxf(s[0], s[1]);
+  const f32x16_t zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  float alpha_prev = 1.0f;  // what O must be multiplied by before the next P V is added
+  // O *= alpha.  The output tile lives in accumulation registers, which the VALU cannot
+  // address; written as plain C++ the allocator copies all 128 of them into VGPRs at the top of
+  // every step, whether or not this rare path runs.  Spelled out, the copies stay in here.
+  auto rescale_output = [&](float alpha) {
+    // the hazard checker does not look inside the statements below: give the last MFMAs time to
+    // retire their results before they are read, and the writes time to land before the next MFMA
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
 #pragma unroll
-    for (int i = 2; i < 16; ++i) m = fmaxf(m, s[i]);
-    return m;
+    for (int dt = 0; dt < kDT; ++dt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        float x = oacc[dt][i], t;
+        asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 %0, %1"
+                     : "+a"(x), "=&v"(t)
+                     : "v"(alpha));
+        oacc[dt][i] = x;
+      }
+    asm volatile("s_nop 7" ::: "memory");
   };
-  auto decide = [&](float mx, Stats& st) {
-    const float m = wave_max_xor(mx * st.mul, 32);
-    const float m_old = m_run;
-    const float m_new = fmaxf(m_old, m);
-    const float m_use = (m_new - m_old > kLazy) ? m_new : m_old;
-    st.m_safe = (m_use == kNegInf) ? 0.f : m_use;
-    st.alpha = fast_exp2(m_old - st.m_safe);
-    m_run = m_use;
-    pin(st.m_safe);
-    pin(st.alpha);
-  };
-  // One step over halves i-1, i, i+1, cut into four slices by scheduling barriers (inside a
-  // slice the compiler interleaves MFMA, LDS reads and VALU freely, across slices nothing
-  // moves).  Matrix pipe: scores of half i+1 in slices 0, 1; P V of half i-1 in slices 2, 3.
-  // VALU: exponentials and packing of half i in slices 0..2; row max and softmax state of half
-  // i+1 in slices 2, 3.  Each slice requests the LDS operands of the next one; slice 3 requests
-  // the first K operands of the next step (`kops`, carried between calls).
-  auto step = [&](f32x16_t& cur, const Stats& st_cur, f32x16_t& nxt, Stats& st_nxt, bool mask_nxt,
-                  int nxt_base, const unsigned char* ks, const unsigned char* vs,
-                  const unsigned char* ks_after, bf16x8_t (&kops)[8], const bf16x8_t (&pb_prev)[2],
-                  bf16x8_t (&pb_cur)[2], uint32_t k_fill, uint32_t v_fill) {
-    float psum = 0.f;
+  // One step over halves i-1, i, i+1.  The 32 MFMAs (16 chained ones for the scores of half
+  // i+1, 16 independent ones adding P V of half i-1) depend on nothing the VALU does in this
+  // step; they are spread over four slices, 4 + 4 each, so that the score chain always has an
+  // independent neighbour, and each slice requests the LDS operands of the next (the last one
+  // those of the next step's first slice: `kq[0]`, `vq[0]` are carried between calls).  The
+  // VALU settles the softmax state of half i (row max against the lazy running max), then
+  // turns its scores into bf16 P and the row sum.  Scheduling barriers separate the slices:
+  // inside one the compiler interleaves freely, across them nothing moves.
+  //   m_safe  the (lazy) running row max the exponentials are taken against
+  //   alpha   exp2(previous max - m_safe): what O and l must be multiplied by first
+  auto step = [&](f32x16_t& cur, f32x16_t& nxt, bool mask_cur, int cur_base, const unsigned char* ks,
+                  const unsigned char* vs, const unsigned char* ks_after, const unsigned char* vs_after,
+                  bf16x8_t (&kq)[2][4], bf16x8_t (&vq)[2][4], const bf16x8_t (&pb_prev)[2],
+                  bf16x8_t (&pb_cur)[2], uint32_t k_fill, uint32_t v_fill, const OffT (&voff)[kUPW]) {
+    if (__any(alpha_prev != 1.0f)) {  // rare: some row's lazy max moved in the previous step
+      rescale_output(alpha_prev);
+    }
+    // softmax scale: applied inside the exponent on interior halves (max commutes with a
+    // positive scale); boundary halves are scaled and masked in place
+    float mul = p.scale_log2e;
+    if (mask_cur) {
+      asm volatile("" ::: "memory");  // keeps this a branch instead of 64 selects in every step
+      mask_in_place(cur, cur_base);
+      mul = 1.0f;
+    }
+    float psum = 0.f, m_safe, alpha;
+    auto settle = [&]() {
+      float mx = fmaxf(cur[0], cur[1]);
+#pragma unroll
+      for (int i = 2; i < 16; ++i) mx = fmaxf(mx, cur[i]);
+      const float m = wave_max_xor(mx * mul, 32);
+      const float m_old = m_run;
+      const float m_new = fmaxf(m_old, m);
+      const float m_use = (m_new - m_old > kLazy) ? m_new : m_old;
+      m_safe = (m_use == kNegInf) ? 0.f : m_use;
+      alpha = fast_exp2(m_old - m_safe);
+      m_run = m_use;
+    };
     auto exp_slice = [&](int first) {  // elements first .. first+7
 #pragma unroll
       for (int i = first; i < first + 8; ++i) {
-        float e = fast_exp2(__builtin_fmaf(cur[i], st_cur.mul, -st_cur.m_safe));
+        float e = fast_exp2(__builtin_fmaf(cur[i], mul, -m_safe));
         pin(e);  // keeps the arithmetic in its slice
         cur[i] = e;
       }
@@ -284,54 +301,66 @@ __global__ __launch_bounds__(kNW * 64) void prefill_tile256_kernel(PrefillParams
       }
       pb_cur[u] = as_bf16x8(pk);
     };
-    auto moves = [&](int slice) {
+    auto mfma_slice = [&](int s) {  // k-steps 4s .. 4s+3 of the scores; keys 16 (s/2).., dim tiles 4 (s%2)..
 #pragma unroll
-      for (int n = slice * 2; n < slice * 2 + 2; ++n) move(n, k_fill, v_fill);
+      for (int e = 0; e < 4; ++e) {
+        nxt = mfma_32x32x16(kq[s & 1][e], qreg[4 * s + e], (s == 0 && e == 0) ? zero16 : nxt);
+        const int dt = 4 * (s & 1) + e;
+        oacc[dt] = mfma_32x32x16(vq[s & 1][e], pb_prev[s >> 1], oacc[dt]);
+      }
     };
-    bf16x8_t ops_a[8], ops_b[8];
+    auto request_slice = [&](int s) {  // LDS operands of slice s (s == 4: slice 0 of the next step)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        kq[s & 1][e] = (s < 4) ? k_operand(ks, 4 * s + e) : k_operand(ks_after, e);
+        vq[s & 1][e] = (s < 4) ? v_operand(vs, s >> 1, 4 * (s & 1) + e) : v_operand(vs_after, 0, e);
+      }
+    };
+    auto moves = [&](int s) {
+#pragma unroll
+      for (int n = s * 2; n < s * 2 + 2; ++n) move(n, k_fill, v_fill, voff);
+    };
+    // Order inside a slice: its 12 LDS requests first, then each of the 8 MFMAs followed by a
+    // share of the slice's VALU work (left alone, the scheduler issues the requests last, and
+    // the next slice starts by waiting for them).
+    auto slice_order = [](auto valu_per_mfma) {
+      __builtin_amdgcn_sched_group_barrier(0x100, 12, 0);  // LDS reads
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                    // MFMA
+        __builtin_amdgcn_sched_group_barrier(0x002, decltype(valu_per_mfma)::value, 0);  // VALU
+      }
+    };
     // slice 0
-#pragma unroll
-    for (int i = 0; i < 16; ++i) nxt[i] = 0.f;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) ops_a[e] = k_operand(ks, 8 + e);
-#pragma unroll
-    for (int e = 0; e < 8; ++e) nxt = mfma_32x32x16(kops[e], qreg[e], nxt);
+    request_slice(1);
+    mfma_slice(0);
+    settle();
     exp_slice(0);
     moves(0);
+    slice_order(std::integral_constant<int, 6>{});
     __builtin_amdgcn_sched_barrier(0);
     // slice 1
-#pragma unroll
-    for (int dt = 0; dt < kDT; ++dt) ops_b[dt] = v_operand(vs, 0, dt);
-#pragma unroll
-    for (int e = 0; e < 8; ++e) nxt = mfma_32x32x16(ops_a[e], qreg[8 + e], nxt);
+    request_slice(2);
+    mfma_slice(1);
     exp_slice(8);
     pack_slice(0);
     moves(1);
+    slice_order(std::integral_constant<int, 5>{});
     __builtin_amdgcn_sched_barrier(0);
-    st_nxt.mul = p.scale_log2e;
-    if (mask_nxt) {  // boundary half: scale and mask in place
-      asm volatile("" ::: "memory");  // keeps this a branch instead of 64 selects in every step
-      mask_in_place(nxt, nxt_base);
-      st_nxt.mul = 1.0f;
-    }
     // slice 2
-#pragma unroll
-    for (int dt = 0; dt < kDT; ++dt) ops_a[dt] = v_operand(vs, 1, dt);
-#pragma unroll
-    for (int dt = 0; dt < kDT; ++dt) oacc[dt] = mfma_32x32x16(ops_b[dt], pb_prev[0], oacc[dt]);
+    request_slice(3);
+    mfma_slice(2);
     pack_slice(1);
-    float mx = lane_max(nxt);
-    pin(mx);
     moves(2);
+    slice_order(std::integral_constant<int, 2>{});
     __builtin_amdgcn_sched_barrier(0);
     // slice 3
-#pragma unroll
-    for (int e = 0; e < 8; ++e) kops[e] = k_operand(ks_after, e);
-#pragma unroll
-    for (int dt = 0; dt < kDT; ++dt) oacc[dt] = mfma_32x32x16(ops_a[dt], pb_prev[1], oacc[dt]);
-    l_run = l_run * st_cur.alpha + psum;
-    decide(mx, st_nxt);
+    request_slice(4);
+    mfma_slice(3);
+    l_run = l_run * alpha + psum;
+    alpha_prev = alpha;
     moves(3);
+    slice_order(std::integral_constant<int, 1>{});
     __builtin_amdgcn_sched_barrier(0);
   };
 
@@ -340,97 +369,74 @@ __global__ __launch_bounds__(kNW * 64) void prefill_tile256_kernel(PrefillParams
     return general_scale || (base < w_lo_max) || (base + 31 > w_hi_min);
   };
   if (n_steps > 0) {
-    // ---- prologue: K of halves 0..3 and V of half 0 leave; the first four stages are waited for
-    Slots sk, sv;
+    // ---- prologue: K of halves 0..3 and V of halves 0, 1 leave; all but K of half 3 are waited
+    // for.  K of half x lives in K stage x % 4, V of half x in V stage x % 4.
+    Slots sl;
 #pragma unroll
-    for (int x = 0; x < 3; ++x) {
-      slot_load(k_lo + x * kHalf, sk);
-      k_offsets(sk);
-      if (x == 0) v_offsets(sk);
+    for (int x = 0; x < 4; ++x) {
+      slot_load(k_lo + x * kHalf, sl);
 #pragma unroll
-      for (int n = (x == 0 ? 0 : kUPW); n < kMovesPerStep; ++n) move(n, x * kKStage, kVBase);
+      for (int i = 0; i < kUPW; ++i) {
+        k_off[i] = lane_offset(sl.s[0][i], sl.s[1][i], k_row_bytes);
+        v_off[x & 1][i] = lane_offset(sl.s[0][i], sl.s[1][i], v_row_bytes);
+      }
+#pragma unroll
+      for (int n = (x < 2 ? 0 : kUPW); n < kMovesPerStep; ++n)
+        move(n, x * kKStage, kVBase + x * kVStage, v_off[x & 1]);
+      // the V offsets of halves 2 and 3 stay in v_off[0], v_off[1] for the moves of steps 0 and 1
     }
-    slot_load(k_lo + 3 * kHalf, sk);
-    k_offsets(sk);
-#pragma unroll
-    for (int n = kUPW; n < kMovesPerStep; ++n) move(n, 3 * kKStage, 0);
-    // slot ids for the moves of step 0: K of half 4, V of half 1
-    slot_load(k_lo + 4 * kHalf, sk);
-    slot_load(k_lo + 1 * kHalf, sv);
+    slot_load(k_lo + 4 * kHalf, sl);  // for the K move of step 0
     wait_vm_at_most<kUPW>();
     __syncthreads();
 
-    f32x16_t sa, sb;
-    Stats st_a, st_b;
+    f32x16_t sa = zero16, sb;
     bf16x8_t pb_a[2], pb_b[2];
     {  // scores of half 0
       const unsigned char* ks = smem + k_lane;
 #pragma unroll
-      for (int i = 0; i < 16; ++i) sa[i] = 0.f;
-#pragma unroll
       for (int kstep = 0; kstep < kKSteps; ++kstep) sa = mfma_32x32x16(k_operand(ks, kstep), qreg[kstep], sa);
     }
-    st_a.mul = p.scale_log2e;
-    if (needs_mask(k_lo)) {
-      mask_in_place(sa, k_lo);
-      st_a.mul = 1.0f;
-    }
-    decide(lane_max(sa), st_a);
-    st_b.mul = 1.0f;
-    st_b.alpha = 1.0f;
-    st_b.m_safe = 0.f;
 #pragma unroll
     for (int u = 0; u < 2; ++u) pb_b[u] = as_bf16x8(u32x4_t{0u, 0u, 0u, 0u});
-
-    // Stage rings.  Step i reads K of half i+1 (stage (i+1) % 4), takes the first operands of
-    // half i+2, fills stage i % 4 with half i+4; reads V of half i-1 (stage (i-1) % 3; the P
-    // of "half -1" is zero, so step 0 may read V of half 0) and fills stage (i+1) % 3.
-    uint32_t kr = 0;              // i % 4
-    uint32_t v_read = kVBase;     // stage of half i-1
-    uint32_t v_mid = kVBase;      // stage of half i (being waited for during step i-1 .. i)
-    uint32_t v_fill = kVBase + kVStage;
-    uint32_t v_free = kVBase + 2 * kVStage;
-    bf16x8_t kops[8];
+    // Step i reads K of half i+1, requests the first operands of half i+2 and fills the stage
+    // of half i with half i+4; it reads V of half i-1 (the P of "half -1" is zero, so step 0
+    // may read V of half 0), requests the first operands of half i and fills the stage of
+    // half i-2 with half i+2.
+    bf16x8_t kq[2][4], vq[2][4];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) kops[e] = k_operand(smem + kKStage + k_lane, e);
-
-    auto k_stage = [&](uint32_t r) { return (r & 3u) * (uint32_t)kKStage; };
-    auto advance = [&](int i) {
-      kr = (kr + 1) & 3u;
-      const uint32_t freed = (i == 0) ? v_free : v_read;
-      v_read = v_mid;
-      v_mid = v_fill;
-      v_fill = freed;
+    for (int e = 0; e < 4; ++e) {
+      kq[0][e] = k_operand(smem + kKStage + k_lane, e);
+      vq[0][e] = v_operand(smem + kVBase + v_lane, 0, e);
+    }
+    auto k_stage = [&](int x) { return (uint32_t)(x & 3) * (uint32_t)kKStage; };
+    auto v_stage = [&](int x) { return (uint32_t)kVBase + (uint32_t)(x & 3) * (uint32_t)kVStage; };
+    auto one_step = [&](int i, f32x16_t& cur, f32x16_t& nxt, const bf16x8_t (&pb_prev)[2],
+                        bf16x8_t (&pb_cur)[2], OffT (&voff)[kUPW]) {
+      const int tb = k_lo + i * kHalf;
+      // offsets of K of half i+4 from the slot ids requested one step ago; the same ids give the
+      // V offsets that half will need two steps from now
+#pragma unroll
+      for (int n = 0; n < kUPW; ++n) k_off[n] = lane_offset(sl.s[0][n], sl.s[1][n], k_row_bytes);
+      OffT v_new[kUPW];
+#pragma unroll
+      for (int n = 0; n < kUPW; ++n) v_new[n] = lane_offset(sl.s[0][n], sl.s[1][n], v_row_bytes);
+      slot_load(tb + 5 * kHalf, sl);
+      step(cur, nxt, needs_mask(tb), tb, smem + k_stage(i + 1) + k_lane,
+           smem + v_stage(i == 0 ? 0 : i - 1) + v_lane, smem + k_stage(i + 2) + k_lane,
+           smem + v_stage(i) + v_lane, kq, vq, pb_prev, pb_cur, k_stage(i), v_stage(i + 2), voff);
+#pragma unroll
+      for (int n = 0; n < kUPW; ++n) voff[n] = v_new[n];
+      wait_vm_at_most<kMovesPerStep>();
+      __syncthreads();
     };
     for (int i = 0; i < n_steps; i += 2) {
-      const int tb = k_lo + i * kHalf;
-      // step i: cur = sa
-      k_offsets(sk);
-      v_offsets(sv);
-      slot_load(tb + 5 * kHalf, sk);
-      slot_load(tb + 2 * kHalf, sv);
-      rescale(st_b.alpha);
-      step(sa, st_a, sb, st_b, needs_mask(tb + kHalf), tb + kHalf, smem + k_stage(kr + 1) + k_lane,
-           smem + v_read + v_lane, smem + k_stage(kr + 2) + k_lane, kops, pb_b, pb_a, k_stage(kr), v_fill);
-      wait_vm_at_most<kMovesPerStep>();
-      __syncthreads();
-      advance(i);
-      // step i+1: cur = sb
-      k_offsets(sk);
-      v_offsets(sv);
-      slot_load(tb + 6 * kHalf, sk);
-      slot_load(tb + 3 * kHalf, sv);
-      rescale(st_a.alpha);
-      step(sb, st_b, sa, st_a, needs_mask(tb + 2 * kHalf), tb + 2 * kHalf, smem + k_stage(kr + 1) + k_lane,
-           smem + v_read + v_lane, smem + k_stage(kr + 2) + k_lane, kops, pb_a, pb_b, k_stage(kr), v_fill);
-      wait_vm_at_most<kMovesPerStep>();
-      __syncthreads();
-      advance(i + 1);
+      one_step(i, sa, sb, pb_b, pb_a, v_off[0]);
+      one_step(i + 1, sb, sa, pb_a, pb_b, v_off[1]);
     }
-    // the last half's P V is still owed: V of half n_steps-1 sits in the stage `v_read`
-    rescale(st_b.alpha);
+    // the last half's P V is still owed
+    if (__any(alpha_prev != 1.0f)) rescale_output(alpha_prev);
     {
-      const unsigned char* vs = smem + v_read + v_lane;
+      const unsigned char* vs = smem + v_stage(n_steps - 1) + v_lane;
 #pragma unroll
       for (int u = 0; u < 2; ++u)
 #pragma unroll

@@ -202,11 +202,14 @@ def _scaled(x: int, scale: float, floor: int = 1) -> int:
 
 
 def config_workload(cfg: int, *, scale: float = 1.0, variant: str = "",
-                    pool_device=None) -> PagedWorkload:
+                    pool_device=None, head_dim: int = 128) -> PagedWorkload:
     """Workload of benchmark shape ``cfg`` (1..5); ``scale`` < 1 shrinks the lengths (and, for
     shape 3, the extend) for CPU-sized tests.  ``variant="window"`` selects the sliding
-    window 1024 run of shape 5.  ``pool_device`` draws the two pools on that device."""
+    window 1024 run of shape 5.  ``pool_device`` draws the two pools on that device.
+    ``head_dim`` other than 128 (shape 3 only) gives the same extend at that head size."""
     g = torch.Generator().manual_seed(SEED_BASE + cfg)
+    if head_dim != 128 and cfg != 3:
+        raise ValueError("head_dim is selectable for shape 3 only")
     if cfg == 1:
         lens = [_scaled(l, scale) for l in (37, 128, 500, 1023)]
         return build_workload("cfg1_decode_qwen3_0.6b", "decode", seed=0, generator=g, n_q=16,
@@ -218,9 +221,11 @@ def config_workload(cfg: int, *, scale: float = 1.0, variant: str = "",
     if cfg == 3:
         ext = _scaled(512, scale)
         prefixes = _randint_list(0, _scaled(16384, scale), 8, g)
-        return build_workload("cfg3_extend_qwen3_8b", "prefill", seed=0, generator=g, n_q=32,
-                              n_kv=8, kv_lens=[p + ext for p in prefixes], extend_lens=[ext] * 8,
-                              pool_factor=1.5, store_new=True, pool_device=pool_device)
+        name = "cfg3_extend_qwen3_8b" + ("" if head_dim == 128 else f"_head_dim_{head_dim}")
+        return build_workload(name, "prefill", seed=0, generator=g, n_q=32, n_kv=8,
+                              head_dim=head_dim, kv_lens=[p + ext for p in prefixes],
+                              extend_lens=[ext] * 8, pool_factor=1.5, store_new=True,
+                              pool_device=pool_device)
     if cfg == 4:
         lens = _randint_list(_scaled(32768, scale), _scaled(131072, scale), 16, g)
         return build_workload("cfg4_decode_qwen3_32b_long", "decode", seed=0, generator=g, n_q=64,
