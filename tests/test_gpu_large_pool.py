@@ -11,19 +11,21 @@ from _util import assert_close_bf16, bf16_randn, indptr
 
 pytestmark = pytest.mark.gpu
 
-N_KV, D = 8, 128
-NUM_SLOTS = (4 << 30) // (N_KV * D * 2) + 4096  # a little over 4 GiB per pool
+N_KV = 8
 
 
-def _spread_slots(n, seed):
+def _spread_slots(n, num_slots, seed):
     g = torch.Generator().manual_seed(seed)
-    s = torch.randperm(NUM_SLOTS - 2, generator=g)[: n - 2] + 1
-    return torch.cat([torch.tensor([NUM_SLOTS - 1, 0]), s]).to(torch.int32)
+    s = torch.randperm(num_slots - 2, generator=g)[: n - 2] + 1
+    return torch.cat([torch.tensor([num_slots - 1, 0]), s]).to(torch.int32)
 
 
-def test_store_decode_and_extend_in_a_pool_over_4gib(gpu):
+@pytest.mark.parametrize("D", [128, 256])
+def test_store_decode_and_extend_in_a_pool_over_4gib(gpu, D):
     from mini_sglang_amd_kernel import (paged_decode_attention, paged_prefill_attention,
                                         store_kv_cache)
+
+    NUM_SLOTS = (4 << 30) // (N_KV * D * 2) + 4096  # a little over 4 GiB per pool
 
     free_b, _ = torch.cuda.mem_get_info()
     if free_b < 12 << 30:
@@ -35,7 +37,7 @@ def test_store_decode_and_extend_in_a_pool_over_4gib(gpu):
     kv_lens = [700, 3, 1500]
     ext = [300, 3, 70]           # extend lengths of the prefill call (tile route: 300*4 rows)
     total = sum(kv_lens)
-    slots = _spread_slots(total, 5)
+    slots = _spread_slots(total, NUM_SLOTS, 5)
     k_rows = bf16_randn((total, N_KV, D), 11)
     v_rows = bf16_randn((total, N_KV, D), 12)
     # every row goes in through the store kernel
