@@ -1,7 +1,9 @@
-"""KV-cache interface of the path (reference: mini_sglang_mlx/kvcache/base.py:11-34)."""
+"""KV-cache and prefix-cache interfaces of the path (reference: mini_sglang_mlx/kvcache/base.py)."""
 from __future__ import annotations
 
 from abc import ABC, abstractmethod
+from dataclasses import dataclass
+from typing import NamedTuple, Tuple
 
 import torch
 
@@ -24,3 +26,46 @@ class BaseKVCache(ABC):
     @property
     @abstractmethod
     def num_layers(self) -> int: ...
+
+
+@dataclass(frozen=True)
+class BaseCacheHandle(ABC):
+    """Reference: mini_sglang_mlx/kvcache/base.py:37-39."""
+    cached_len: int
+
+
+class SizeInfo(NamedTuple):
+    """Reference: mini_sglang_mlx/kvcache/base.py:42-48."""
+    evictable_size: int
+    protected_size: int
+
+    @property
+    def total_size(self) -> int:
+        return self.evictable_size + self.protected_size
+
+
+class BaseCacheManager(ABC):
+    """Prefix-cache interface (mini_sglang_mlx/kvcache/base.py:51-121).  ``input_ids`` and
+    ``indices`` are 1-D int32 tensors; what comes back lives in host memory."""
+
+    @abstractmethod
+    def match_prefix(self, input_ids: torch.Tensor) -> Tuple[BaseCacheHandle, torch.Tensor]: ...
+
+    @abstractmethod
+    def lock_handle(self, handle: BaseCacheHandle, unlock: bool = False) -> None: ...
+
+    @abstractmethod
+    def insert_prefix(self, input_ids: torch.Tensor, indices: torch.Tensor) -> int: ...
+
+    @abstractmethod
+    def evict(self, size: int) -> torch.Tensor: ...
+
+    @abstractmethod
+    def reset(self) -> None: ...
+
+    @property
+    @abstractmethod
+    def size_info(self) -> SizeInfo: ...
+
+    @abstractmethod
+    def check_integrity(self) -> None: ...

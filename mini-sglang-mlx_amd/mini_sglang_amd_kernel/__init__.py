@@ -21,7 +21,8 @@ import torch
 from . import _lib
 
 __all__ = ["store_kv_cache", "paged_decode_attention", "paged_prefill_attention",
-           "build_attention_metadata", "qk_norm_rope_store", "gdn_state_inplace"]
+           "build_attention_metadata", "qk_norm_rope_store", "gdn_state_inplace",
+           "fast_compare_key"]
 
 _DTYPE_CODE = {torch.bfloat16: _lib.MSGL_DTYPE_BF16, torch.float16: _lib.MSGL_DTYPE_F16}
 
@@ -443,3 +444,25 @@ def gdn_state_inplace(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torc
         1 if single_token_mode else 0, _stream_ptr(stream, dev))
     _check_rc(op, rc)
     return y
+
+
+def fast_compare_key(a: torch.Tensor, b: torch.Tensor) -> int:
+    """Length of the common prefix of two 1-D integer arrays (host tensors).
+
+    Drop-in for ``mini_sglang_mlx_kernel.fast_compare_key`` (fast_compare_key.cpp:9-45): the
+    radix tree's key comparison.  Pure host code; device tensors are refused instead of being
+    copied behind the caller's back.
+    """
+    op = "fast_compare_key"
+    if a.dim() != 1 or b.dim() != 1:
+        _fail(op, "Both arrays must be 1D.")
+    if not a.is_contiguous() or not b.is_contiguous():
+        _fail(op, "Both arrays must be contiguous.")
+    if a.dtype != b.dtype:
+        _fail(op, "Both arrays must have the same dtype.")
+    if a.dtype not in (torch.int32, torch.int64):
+        _fail(op, "Arrays must be int32 or int64.")
+    if a.device.type != "cpu" or b.device.type != "cpu":
+        _fail(op, "Both arrays must live in host memory.")
+    return int(_lib.load().msgl_fast_compare_key(a.data_ptr(), a.numel(), b.data_ptr(), b.numel(),
+                                                 a.element_size(), None))

@@ -1,4 +1,5 @@
-"""ctypes binding of ``libmsgl_paged_attention.so`` (the C ABI in ``include/msgl_paged_attention.h``).
+"""ctypes binding of ``libmsgl_paged_attention.so`` (the C ABI in ``include/msgl_paged_attention.h``
+and ``include/msgl_radix_cache.h``).
 
 The library is built in-tree by ``mini-sglang-mlx_amd/build.py``; nothing here compiles at
 import time and nothing falls back to another implementation: a missing library is an
@@ -18,7 +19,7 @@ _f32 = ctypes.c_float
 _vp = ctypes.c_void_p
 _sz = ctypes.c_size_t
 
-# name -> (restype, argtypes); one entry per MSGL_API declaration of the header
+# name -> (restype, argtypes); one entry per MSGL_API declaration of the headers
 SIGNATURES = {
     "msgl_version": (ctypes.c_int, []),
     "msgl_strerror": (ctypes.c_char_p, [ctypes.c_int]),
@@ -48,6 +49,26 @@ SIGNATURES = {
         ctypes.c_int,
         [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64,
          _i64, _i64, _i64, _i64, _i32, _vp]),
+    # include/msgl_radix_cache.h (host-side prefix cache)
+    "msgl_fast_compare_key": (_sz, [_vp, _sz, _vp, _sz, _i32, _vp]),
+    "msgl_radix_create": (_vp, []),
+    "msgl_radix_destroy": (None, [_vp]),
+    "msgl_radix_walk": (_i64, [_vp, _vp, _i64, _i64, _vp]),
+    "msgl_radix_path_values": (_i64, [_vp, _i64, _vp, _i64]),
+    "msgl_radix_insert": (_i64, [_vp, _vp, _vp, _i64, _i32, _i64, _vp]),
+    "msgl_radix_lock": (_i32, [_vp, _i64, _i32]),
+    "msgl_radix_evict": (_i64, [_vp, _i64, _i64, _vp]),
+    "msgl_radix_evicted": (_i32, [_vp, _vp, _i64, _vp, _i64]),
+    "msgl_radix_sizes": (_i32, [_vp, _vp, _vp]),
+    "msgl_radix_node_info": (_i32, [_vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "msgl_radix_node_set": (_i32, [_vp, _i64, _i32, _i64]),
+    "msgl_radix_node_child": (_i64, [_vp, _i64, _i32]),
+    "msgl_radix_node_children": (_i64, [_vp, _i64, _vp, _vp, _i64]),
+    "msgl_radix_node_key_value": (_i64, [_vp, _i64, _vp, _vp, _i64]),
+    "msgl_radix_find_mamba_ancestor": (_i64, [_vp, _i64, _i64, _vp]),
+    "msgl_radix_collect_mamba_slots": (_i64, [_vp, _vp, _i64]),
+    "msgl_radix_coldest_snapshot": (_i64, [_vp, _i64]),
+    "msgl_radix_node_count": (_i64, [_vp]),
 }
 
 MSGL_DTYPE_BF16 = 0

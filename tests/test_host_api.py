@@ -12,11 +12,12 @@ import pytest
 import torch
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-HEADER = os.path.join(ROOT, "include", "msgl_paged_attention.h")
+HEADERS = sorted(os.path.join(ROOT, "include", f) for f in os.listdir(os.path.join(ROOT, "include"))
+                 if f.endswith(".h"))
 
 
 def _declared_symbols():
-    text = open(HEADER).read()
+    text = "\n".join(open(h).read() for h in HEADERS)
     return sorted(set(re.findall(r"MSGL_API\s+[\w\s\*]+?\b(msgl_\w+)\s*\(", text)))
 
 
