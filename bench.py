@@ -371,6 +371,62 @@ def run_gdn_state(dev, steps: int, warmup: int, cpu_baseline: bool):
     return rows_out
 
 
+def run_radix_cache(cpu_baseline: bool):
+    """Host-side prefix cache: 2048 finished requests (one of 8 shared 1024-token system prompts
+    plus a 512-token body of their own) are inserted, then every request comes back with 64 new
+    tokens and is matched.  Timed with the host clock; no GPU work.  The same trace through the
+    pure-Python oracle (a quarter of it) is the CPU baseline."""
+    import torch
+
+    from mini_sglang_amd.kvcache import RadixCacheManager
+
+    g = torch.Generator().manual_seed(0x5EED0200)
+    prompts = torch.randint(0, 150000, (8, 1024), generator=g, dtype=torch.int32)
+    bodies = torch.randint(0, 150000, (2048, 512 + 64), generator=g, dtype=torch.int32)
+    which = torch.randint(0, 8, (2048,), generator=g)
+    seqs = [torch.cat([prompts[int(which[i])], bodies[i]]) for i in range(2048)]
+    pages = torch.arange(1536, dtype=torch.int32)
+
+    def trace(insert, match, n):
+        t0 = time.perf_counter()
+        for i in range(n):
+            insert(seqs[i][:1536], pages)
+        t1 = time.perf_counter()
+        hit = 0
+        for i in range(n):
+            hit += match(seqs[i])
+        t2 = time.perf_counter()
+        return (t1 - t0) / n, (t2 - t1) / n, hit / n
+
+    mgr = RadixCacheManager()
+    ins_s, match_s, hit = trace(mgr.insert_prefix, lambda s: mgr.match_prefix(s)[0].cached_len, 2048)
+    row = {"requests": 2048, "tokens_per_request": 1536, "insert_us": ins_s * 1e6,
+           "match_us": match_s * 1e6, "mean_cached_len": hit,
+           "match_tokens_per_s": 1600 / match_s}
+    if cpu_baseline:
+        from oracle.radix_oracle import RadixOracle  # checker and CPU baseline only
+
+        ora = RadixOracle(time.monotonic_ns)
+        lists = [s.tolist() for s in seqs[:512]]
+        page_list = pages.tolist()
+        t0 = time.perf_counter()
+        for ids in lists:
+            ora.insert_prefix(ids[:1536], page_list)
+        t1 = time.perf_counter()
+        hit_o = sum(ora.match_prefix(ids)[0] for ids in lists)
+        t2 = time.perf_counter()
+        row["cpu_port_insert_us"] = (t1 - t0) / 512 * 1e6
+        row["cpu_port_match_us"] = (t2 - t1) / 512 * 1e6
+        row["cpu_port_sample"] = "first 512 requests, pure-Python oracle on lists, 1 core"
+        row["agrees_with_oracle"] = bool(
+            hit_o == sum(RadixCacheManager.match_prefix(mgr, s)[0].cached_len for s in seqs[:512]))
+    log(f"[radix cache] insert {row['insert_us']:.1f} us  match {row['match_us']:.1f} us per request "
+        f"(cached {hit:.0f} of 1600 tokens)  cpu port insert "
+        f"{row.get('cpu_port_insert_us', float('nan')):.0f} us match "
+        f"{row.get('cpu_port_match_us', float('nan')):.0f} us")
+    return row
+
+
 def mfma_rate_probe():
     """Sustained v_mfma_f32_32x32x16_bf16 rate of the whole chip on register-resident operands,
     nothing else running: all-zero operands and N(0,1) operands that change every instruction.
@@ -523,6 +579,7 @@ def main():
                                                     not args.no_cpu_baseline)
         result["metadata_build"] = run_metadata_build(dev, args.steps, args.warmup,
                                                       not args.no_cpu_baseline)
+        result["radix_prefix_cache"] = run_radix_cache(not args.no_cpu_baseline)
     result["all_configs"] = rows
     print(json.dumps(result))
 
