@@ -14,10 +14,12 @@
 //                fall into different banks.
 //   pipeline   = one step per 32 keys: the matrix pipe computes the scores of half i+1 and adds
 //                P V of half i-1 (32 MFMAs) while the VALU turns the scores of half i into P.
-//                K of half i+4 and V of half i+1 leave during step i; a wave waits at the end of
+//                K of half i+4 and V of half i+2 leave during step i; a wave waits at the end of
 //                step i for the moves it issued in step i-1 (vmcnt counts the newer ones), then
 //                the workgroup barrier publishes them: a move has between one and two steps to
-//                land.  Four K stages and three V stages of LDS.
+//                land, and every stage is published a step before its first operand is
+//                requested (the last slice of a step requests the first operands of the next).
+//                Four K stages and four V stages of LDS.
 //   slot ids   = read through the scalar cache (uniform addresses in the constant address
 //                space), so that the only vector-memory operations of a step are its 8 moves
 //                and the counted wait means what it says.
