@@ -1,0 +1,78 @@
+"""Seeded random shapes through both attention operators against the oracle: head counts,
+head sizes, page sizes, ragged lengths (empty requests, single tokens, lengths around the 16-,
+32- and 64-key tile edges), every mask, with and without a store first.  The fixed cases of the
+other modules aim at known edges; this one looks for the ones nobody thought of."""
+import random
+
+import pytest
+import torch
+
+from _gpu_util import run_gpu, run_oracle
+from _util import assert_close_bf16
+from mini_sglang_amd.workloads import build_workload
+
+pytestmark = pytest.mark.gpu
+
+HEADS = [(1, 1), (2, 1), (4, 4), (6, 3), (8, 2), (8, 8), (12, 4), (16, 1), (16, 8), (20, 4), (32, 8)]
+EDGES = [0, 1, 2, 15, 16, 17, 31, 32, 33, 47, 63, 64, 65, 95, 96, 97, 127, 128, 129, 255, 257]
+
+
+def _length(rng, hi):
+    return rng.choice(EDGES) if rng.random() < 0.5 else rng.randrange(0, hi)
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_prefill_shapes(gpu, seed):
+    rng = random.Random(1000 + seed)
+    n_q, n_kv = rng.choice(HEADS)
+    d = rng.choice([128, 128, 256])
+    batch = rng.randrange(1, 6)
+    # short query blocks (split-K route), long ones (tile kernels), and mixtures of both
+    style = rng.choice(["short", "long", "mixed"])
+    ext, kv = [], []
+    for _ in range(batch):
+        if style == "short" or (style == "mixed" and rng.random() < 0.5):
+            e = rng.randrange(0, 9)
+        else:
+            e = max(1, _length(rng, 300))
+        prefix = _length(rng, 700) if rng.random() < 0.8 else 0
+        ext.append(e)
+        kv.append(prefix + e)
+    if sum(ext) == 0:
+        ext[0], kv[0] = 1, kv[0] + 1
+    is_cross = rng.random() < 0.3
+    window = rng.choice([0, 0, 1, 2, 17, 64, 100, 1000])
+    page = rng.choice([1, 4, 16])
+    wl = build_workload("fuzz", "prefill", seed=seed, n_q=n_q, n_kv=n_kv, head_dim=d, page_size=page,
+                        kv_lens=kv, extend_lens=ext, pool_factor=rng.choice([1.0, 1.7]),
+                        store_new=rng.random() < 0.7, is_cross_attention=is_cross,
+                        sliding_window_size=window)
+    what = (f"fuzz prefill seed={seed} heads={n_q}/{n_kv} d={d} page={page} ext={ext} kv={kv} "
+            f"cross={is_cross} W={window}")
+    print(what, flush=True)
+    got, g = run_gpu(wl, gpu)
+    want, ref = run_oracle(wl)
+    assert_close_bf16(got, want, what)
+    if wl.out_loc is not None:
+        assert torch.equal(g.k_cache.cpu().view(torch.int16), ref.k_cache.view(torch.int16)), what
+        assert torch.equal(g.v_cache.cpu().view(torch.int16), ref.v_cache.view(torch.int16)), what
+
+
+@pytest.mark.parametrize("seed", range(25))
+def test_random_decode_shapes(gpu, seed):
+    rng = random.Random(2000 + seed)
+    n_q, n_kv = rng.choice([h for h in HEADS if h[0] // h[1] <= 16])
+    d = rng.choice([128, 128, 256])
+    batch = rng.randrange(1, 40)
+    kv = [_length(rng, 2500) for _ in range(batch)]
+    page = rng.choice([1, 16])
+    wl = build_workload("fuzz", "decode", seed=seed, n_q=n_q, n_kv=n_kv, head_dim=d, page_size=page,
+                        kv_lens=kv, pool_factor=rng.choice([1.0, 1.4]))
+    what = f"fuzz decode seed={seed} heads={n_q}/{n_kv} d={d} page={page} batch={batch} total={sum(kv)}"
+    print(what, flush=True)
+    got, _ = run_gpu(wl, gpu)
+    want, _ = run_oracle(wl)
+    assert_close_bf16(got, want, what)
+    for b, l in enumerate(kv):
+        if l == 0:
+            assert torch.count_nonzero(got[b]) == 0, what
