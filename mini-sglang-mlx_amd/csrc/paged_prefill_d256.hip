@@ -20,9 +20,9 @@
 //                land, and every stage is published a step before its first operand is
 //                requested (the last slice of a step requests the first operands of the next).
 //                Four K stages and four V stages of LDS.
-//   slot ids   = read through the scalar cache (uniform addresses in the constant address
-//                space), so that the only vector-memory operations of a step are its 8 moves
-//                and the counted wait means what it says.
+//   slot ids   = fetched a step ahead by loads issued before the step's moves and hidden from
+//                the compiler's wait bookkeeping, so that the counted wait at the end of the
+//                step (all but the 8 newest operations) covers them and nothing else waits.
 //
 // Algorithmic flops: 4 * D per visible (query, key) pair and q head (QK^T + PV).
 #include <type_traits>
@@ -50,8 +50,6 @@ constexpr int kStageTotal = kVBase + kVStages * kVStage;  // 136192
 constexpr int kKSteps = kD / 16;              // k-steps of QK^T
 constexpr int kDT = kD / 32;                  // 32-dim tiles of O^T
 constexpr int kMovesPerStep = 2 * kUPW;       // V units then K units, per wave
-
-typedef const __attribute__((address_space(4))) int32_t* ConstI32Ptr;
 
 template <bool WIDE>
 __global__ __launch_bounds__(kNW * 64) void prefill_tile256_kernel(PrefillParams p) {
@@ -155,34 +153,42 @@ __global__ __launch_bounds__(kNW * 64) void prefill_tile256_kernel(PrefillParams
   // ---- moving a stage: wave w owns units 4w .. 4w+3; in a unit, lane l fetches 16-byte chunk
   // l % 32 of key (unit + 16 (l / 32)) ----------------------------------------------------
   const uint32_t lds0 = (uint32_t)(uintptr_t)MSGL_LDS_PTR(unsigned char, smem);
-  const ConstI32Ptr idx_base = (ConstI32Ptr)(uintptr_t)(p.kv_indices + kv_start);
   const unsigned char* k_src = reinterpret_cast<const unsigned char*>(p.k_cache + (int64_t)kvh * kD);
   const unsigned char* v_src = reinterpret_cast<const unsigned char*>(p.v_cache + (int64_t)kvh * kD);
   const uint32_t k_row_bytes = (uint32_t)p.k_stride0 * 2u;
   const uint32_t v_row_bytes = (uint32_t)p.v_stride0 * 2u;
   const uint32_t chunk_off = (uint32_t)(lane & 31) * 16u;
-  const bool upper = lane >= 32;
-  struct Slots {
-    int32_t s[2][kUPW];  // slot ids of this wave's keys: [0] keys 4w+i, [1] keys 4w+i+16 (uniform)
-  };
-  // slot ids of the half starting at key `base`: two 16-byte scalar loads when the half lies
-  // inside the request, element-wise clamped loads on its last, partial half
-  auto slot_load = [&](int base, Slots& sl) {
-    const int first = base + w * kUPW;
-    if (first + 16 + kUPW <= kn) {
-#pragma unroll
-      for (int r = 0; r < 2; ++r)
-#pragma unroll
-        for (int i = 0; i < kUPW; ++i) sl.s[r][i] = idx_base[first + 16 * r + i];
+  // Slot ids of a half: lane l wants the ids of keys 4w .. 4w+3 (+16 for the upper half of the
+  // wave).  They are fetched by vector loads the compiler does not see (it would answer the
+  // first use of their result with a wait for every load in flight, the moves included); the
+  // caller's next counted wait, which names the result registers, makes them valid.  One 16-byte
+  // load when the half lies inside the request, element-wise clamped loads on its last,
+  // partial half.
+  const int32_t* idx_ptr = p.kv_indices + kv_start;
+  const int lane_key = w * kUPW + 16 * (lane >> 5);
+  auto slot_load = [&](int base, u32x4_t& sl) {
+    const int first = base + lane_key;
+    if (base + (kNW - 1) * kUPW + 16 + kUPW <= kn) {  // uniform: the whole half is in range
+      const uint32_t off = (uint32_t)first * 4u;
+      asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(sl) : "v"(off), "s"(idx_ptr) : "memory");
     } else {
+      uint32_t e[kUPW];
 #pragma unroll
-      for (int r = 0; r < 2; ++r)
-#pragma unroll
-        for (int i = 0; i < kUPW; ++i) sl.s[r][i] = idx_base[min(first + 16 * r + i, kn - 1)];
+      for (int i = 0; i < kUPW; ++i) {
+        const uint32_t off = (uint32_t)min(first + i, kn - 1) * 4u;
+        asm volatile("global_load_dword %0, %1, %2" : "=v"(e[i]) : "v"(off), "s"(idx_ptr) : "memory");
+      }
+      sl = u32x4_t{e[0], e[1], e[2], e[3]};
     }
   };
-  auto lane_offset = [&](int32_t s_lo, int32_t s_hi, uint32_t row_bytes) -> OffT {
-    const uint32_t slot = (uint32_t)(upper ? s_hi : s_lo);
+  // s_waitcnt vmcnt(N) that also stands for "these slot ids have arrived": nothing that reads
+  // them can be scheduled above it
+  auto wait_vm_and_slots = [&](auto n, u32x4_t& sl) {
+    constexpr int N = decltype(n)::value;
+    static_assert(N >= 0 && N < 16, "low bits of vmcnt only");
+    asm volatile("s_waitcnt vmcnt(%1)" : "+v"(sl) : "n"(N) : "memory");
+  };
+  auto lane_offset = [&](uint32_t slot, uint32_t row_bytes) -> OffT {
     if constexpr (WIDE) return (uint64_t)slot * row_bytes + chunk_off;
     else return __umul24(slot, row_bytes) + chunk_off;  // both factors below 2^24 here
   };
@@ -245,48 +251,56 @@ __global__ __launch_bounds__(kNW * 64) void prefill_tile256_kernel(PrefillParams
       }
     asm volatile("s_nop 7" ::: "memory");
   };
+  // Softmax state of one half, decided as soon as its scores exist:
+  //   mul     factor still to be applied to the scores: the softmax scale on interior halves
+  //           (max commutes with a positive scale), 1 on boundary halves, which are scaled and
+  //           masked in place
+  //   m_safe  the (lazy) running row max the exponentials are taken against
+  //   alpha   exp2(previous max - m_safe): what O and l must be multiplied by first
+  struct Stats {
+    float mul, m_safe, alpha;
+  };
+  auto settle = [&](f32x16_t& s, bool mask, int base, Stats& st) {
+    st.mul = p.scale_log2e;
+    if (mask) {  // boundary half
+      asm volatile("" ::: "memory");  // keeps this a branch instead of 64 selects in every step
+      mask_in_place(s, base);
+      st.mul = 1.0f;
+    }
+    float mx = fmaxf(s[0], s[1]);
+#pragma unroll
+    for (int i = 2; i < 16; ++i) mx = fmaxf(mx, s[i]);
+    const float m = wave_max_xor(mx * st.mul, 32);
+    const float m_old = m_run;
+    const float m_new = fmaxf(m_old, m);
+    const float m_use = (m_new - m_old > kLazy) ? m_new : m_old;
+    st.m_safe = (m_use == kNegInf) ? 0.f : m_use;
+    st.alpha = fast_exp2(m_old - st.m_safe);
+    m_run = m_use;
+  };
   // One step over halves i-1, i, i+1.  The 32 MFMAs (16 chained ones for the scores of half
   // i+1, 16 independent ones adding P V of half i-1) depend on nothing the VALU does in this
   // step; they are spread over four slices, 4 + 4 each, so that the score chain always has an
   // independent neighbour, and each slice requests the LDS operands of the next (the last one
   // those of the next step's first slice: `kq[0]`, `vq[0]` are carried between calls).  The
-  // VALU settles the softmax state of half i (row max against the lazy running max), then
-  // turns its scores into bf16 P and the row sum.  Scheduling barriers separate the slices:
-  // inside one the compiler interleaves freely, across them nothing moves.
-  //   m_safe  the (lazy) running row max the exponentials are taken against
-  //   alpha   exp2(previous max - m_safe): what O and l must be multiplied by first
-  auto step = [&](f32x16_t& cur, f32x16_t& nxt, bool mask_cur, int cur_base, const unsigned char* ks,
+  // VALU turns the scores of half i into bf16 P and the row sum (slices 0..2); in the last
+  // slice the score chain of half i+1 ends first and its softmax state is settled behind the
+  // four P V MFMAs that remain, so the next step starts exponentiating at once.  Scheduling
+  // barriers separate the slices: inside one the compiler interleaves freely, across them
+  // nothing moves.
+  auto step = [&](f32x16_t& cur, const Stats& st_cur, f32x16_t& nxt, Stats& st_nxt, bool mask_nxt,
+                  int nxt_base, const unsigned char* ks,
                   const unsigned char* vs, const unsigned char* ks_after, const unsigned char* vs_after,
                   bf16x8_t (&kq)[2][4], bf16x8_t (&vq)[2][4], const bf16x8_t (&pb_prev)[2],
                   bf16x8_t (&pb_cur)[2], uint32_t k_fill, uint32_t v_fill, const OffT (&voff)[kUPW]) {
     if (__any(alpha_prev != 1.0f)) {  // rare: some row's lazy max moved in the previous step
       rescale_output(alpha_prev);
     }
-    // softmax scale: applied inside the exponent on interior halves (max commutes with a
-    // positive scale); boundary halves are scaled and masked in place
-    float mul = p.scale_log2e;
-    if (mask_cur) {
-      asm volatile("" ::: "memory");  // keeps this a branch instead of 64 selects in every step
-      mask_in_place(cur, cur_base);
-      mul = 1.0f;
-    }
-    float psum = 0.f, m_safe, alpha;
-    auto settle = [&]() {
-      float mx = fmaxf(cur[0], cur[1]);
-#pragma unroll
-      for (int i = 2; i < 16; ++i) mx = fmaxf(mx, cur[i]);
-      const float m = wave_max_xor(mx * mul, 32);
-      const float m_old = m_run;
-      const float m_new = fmaxf(m_old, m);
-      const float m_use = (m_new - m_old > kLazy) ? m_new : m_old;
-      m_safe = (m_use == kNegInf) ? 0.f : m_use;
-      alpha = fast_exp2(m_old - m_safe);
-      m_run = m_use;
-    };
+    float psum = 0.f;
     auto exp_slice = [&](int first) {  // elements first .. first+7
 #pragma unroll
       for (int i = first; i < first + 8; ++i) {
-        float e = fast_exp2(__builtin_fmaf(cur[i], mul, -m_safe));
+        float e = fast_exp2(__builtin_fmaf(cur[i], st_cur.mul, -st_cur.m_safe));
         pin(e);  // keeps the arithmetic in its slice
         cur[i] = e;
       }
@@ -303,10 +317,14 @@ __global__ __launch_bounds__(kNW * 64) void prefill_tile256_kernel(PrefillParams
       }
       pb_cur[u] = as_bf16x8(pk);
     };
-    auto mfma_slice = [&](int s) {  // k-steps 4s .. 4s+3 of the scores; keys 16 (s/2).., dim tiles 4 (s%2)..
+    auto qk_mfmas = [&](int s) {  // k-steps 4s .. 4s+3 of the scores
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        nxt = mfma_32x32x16(kq[s & 1][e], qreg[4 * s + e], (s == 0 && e == 0) ? zero16 : nxt);
+    };
+    auto pv_mfmas = [&](int s) {  // keys 16 (s/2) .. +15, dim tiles 4 (s%2) .. +3
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        nxt = mfma_32x32x16(kq[s & 1][e], qreg[4 * s + e], (s == 0 && e == 0) ? zero16 : nxt);
         const int dt = 4 * (s & 1) + e;
         oacc[dt] = mfma_32x32x16(vq[s & 1][e], pb_prev[s >> 1], oacc[dt]);
       }
@@ -335,15 +353,16 @@ __global__ __launch_bounds__(kNW * 64) void prefill_tile256_kernel(PrefillParams
     };
     // slice 0
     request_slice(1);
-    mfma_slice(0);
-    settle();
+    qk_mfmas(0);
+    pv_mfmas(0);
     exp_slice(0);
     moves(0);
-    slice_order(std::integral_constant<int, 6>{});
+    slice_order(std::integral_constant<int, 4>{});
     __builtin_amdgcn_sched_barrier(0);
     // slice 1
     request_slice(2);
-    mfma_slice(1);
+    qk_mfmas(1);
+    pv_mfmas(1);
     exp_slice(8);
     pack_slice(0);
     moves(1);
@@ -351,18 +370,22 @@ __global__ __launch_bounds__(kNW * 64) void prefill_tile256_kernel(PrefillParams
     __builtin_amdgcn_sched_barrier(0);
     // slice 2
     request_slice(3);
-    mfma_slice(2);
+    qk_mfmas(2);
+    pv_mfmas(2);
     pack_slice(1);
     moves(2);
     slice_order(std::integral_constant<int, 2>{});
     __builtin_amdgcn_sched_barrier(0);
-    // slice 3
+    // slice 3: the end of the score chain first ...
     request_slice(4);
-    mfma_slice(3);
-    l_run = l_run * alpha + psum;
-    alpha_prev = alpha;
+    qk_mfmas(3);
     moves(3);
-    slice_order(std::integral_constant<int, 1>{});
+    __builtin_amdgcn_sched_barrier(0);
+    // ... then the state of half i+1 behind the last P V MFMAs
+    pv_mfmas(3);
+    settle(nxt, mask_nxt, nxt_base, st_nxt);
+    l_run = l_run * st_cur.alpha + psum;
+    alpha_prev = st_cur.alpha;
     __builtin_amdgcn_sched_barrier(0);
   };
 
@@ -373,22 +396,24 @@ __global__ __launch_bounds__(kNW * 64) void prefill_tile256_kernel(PrefillParams
   if (n_steps > 0) {
     // ---- prologue: K of halves 0..3 and V of halves 0, 1 leave; all but K of half 3 are waited
     // for.  K of half x lives in K stage x % 4, V of half x in V stage x % 4.
-    Slots sl;
+    u32x4_t sl;
 #pragma unroll
     for (int x = 0; x < 4; ++x) {
       slot_load(k_lo + x * kHalf, sl);
+      wait_vm_and_slots(std::integral_constant<int, 0>{}, sl);
 #pragma unroll
       for (int i = 0; i < kUPW; ++i) {
-        k_off[i] = lane_offset(sl.s[0][i], sl.s[1][i], k_row_bytes);
-        v_off[x & 1][i] = lane_offset(sl.s[0][i], sl.s[1][i], v_row_bytes);
+        k_off[i] = lane_offset(sl[i], k_row_bytes);
+        v_off[x & 1][i] = lane_offset(sl[i], v_row_bytes);
       }
 #pragma unroll
       for (int n = (x < 2 ? 0 : kUPW); n < kMovesPerStep; ++n)
         move(n, x * kKStage, kVBase + x * kVStage, v_off[x & 1]);
       // the V offsets of halves 2 and 3 stay in v_off[0], v_off[1] for the moves of steps 0 and 1
     }
-    slot_load(k_lo + 4 * kHalf, sl);  // for the K move of step 0
-    wait_vm_at_most<kUPW>();
+    // everything but K of half 3 has to have landed; the ids for the K move of step 0 ride along
+    slot_load(k_lo + 4 * kHalf, sl);
+    wait_vm_and_slots(std::integral_constant<int, 0>{}, sl);
     __syncthreads();
 
     f32x16_t sa = zero16, sb;
@@ -398,6 +423,8 @@ __global__ __launch_bounds__(kNW * 64) void prefill_tile256_kernel(PrefillParams
 #pragma unroll
       for (int kstep = 0; kstep < kKSteps; ++kstep) sa = mfma_32x32x16(k_operand(ks, kstep), qreg[kstep], sa);
     }
+    Stats st_a, st_b;
+    settle(sa, needs_mask(k_lo), k_lo, st_a);
 #pragma unroll
     for (int u = 0; u < 2; ++u) pb_b[u] = as_bf16x8(u32x4_t{0u, 0u, 0u, 0u});
     // Step i reads K of half i+1, requests the first operands of half i+2 and fills the stage
@@ -412,28 +439,28 @@ __global__ __launch_bounds__(kNW * 64) void prefill_tile256_kernel(PrefillParams
     }
     auto k_stage = [&](int x) { return (uint32_t)(x & 3) * (uint32_t)kKStage; };
     auto v_stage = [&](int x) { return (uint32_t)kVBase + (uint32_t)(x & 3) * (uint32_t)kVStage; };
-    auto one_step = [&](int i, f32x16_t& cur, f32x16_t& nxt, const bf16x8_t (&pb_prev)[2],
-                        bf16x8_t (&pb_cur)[2], OffT (&voff)[kUPW]) {
+    auto one_step = [&](int i, f32x16_t& cur, const Stats& st_cur, f32x16_t& nxt, Stats& st_nxt,
+                        const bf16x8_t (&pb_prev)[2], bf16x8_t (&pb_cur)[2], OffT (&voff)[kUPW]) {
       const int tb = k_lo + i * kHalf;
       // offsets of K of half i+4 from the slot ids requested one step ago; the same ids give the
       // V offsets that half will need two steps from now
 #pragma unroll
-      for (int n = 0; n < kUPW; ++n) k_off[n] = lane_offset(sl.s[0][n], sl.s[1][n], k_row_bytes);
+      for (int n = 0; n < kUPW; ++n) k_off[n] = lane_offset(sl[n], k_row_bytes);
       OffT v_new[kUPW];
 #pragma unroll
-      for (int n = 0; n < kUPW; ++n) v_new[n] = lane_offset(sl.s[0][n], sl.s[1][n], v_row_bytes);
-      slot_load(tb + 5 * kHalf, sl);
-      step(cur, nxt, needs_mask(tb), tb, smem + k_stage(i + 1) + k_lane,
+      for (int n = 0; n < kUPW; ++n) v_new[n] = lane_offset(sl[n], v_row_bytes);
+      slot_load(tb + 5 * kHalf, sl);  // issued before this step's moves: older than all of them
+      step(cur, st_cur, nxt, st_nxt, needs_mask(tb + kHalf), tb + kHalf, smem + k_stage(i + 1) + k_lane,
            smem + v_stage(i == 0 ? 0 : i - 1) + v_lane, smem + k_stage(i + 2) + k_lane,
            smem + v_stage(i) + v_lane, kq, vq, pb_prev, pb_cur, k_stage(i), v_stage(i + 2), voff);
 #pragma unroll
       for (int n = 0; n < kUPW; ++n) voff[n] = v_new[n];
-      wait_vm_at_most<kMovesPerStep>();
+      wait_vm_and_slots(std::integral_constant<int, kMovesPerStep>{}, sl);
       __syncthreads();
     };
     for (int i = 0; i < n_steps; i += 2) {
-      one_step(i, sa, sb, pb_b, pb_a, v_off[0]);
-      one_step(i + 1, sb, sa, pb_a, pb_b, v_off[1]);
+      one_step(i, sa, st_a, sb, st_b, pb_b, pb_a, v_off[0]);
+      one_step(i + 1, sb, st_b, sa, st_a, pb_a, pb_b, v_off[1]);
     }
     // the last half's P V is still owed
     if (__any(alpha_prev != 1.0f)) rescale_output(alpha_prev);
