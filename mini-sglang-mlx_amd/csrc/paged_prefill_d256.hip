@@ -396,24 +396,30 @@ __global__ __launch_bounds__(kNW * 64) void prefill_tile256_kernel(PrefillParams
   if (n_steps > 0) {
     // ---- prologue: K of halves 0..3 and V of halves 0, 1 leave; all but K of half 3 are waited
     // for.  K of half x lives in K stage x % 4, V of half x in V stage x % 4.
-    u32x4_t sl;
+    u32x4_t sl, first_slots[4];
+#pragma unroll
+    for (int x = 0; x < 4; ++x) slot_load(k_lo + x * kHalf, first_slots[x]);
+    slot_load(k_lo + 4 * kHalf, sl);  // for the K move of step 0
+    // one round trip for all five (the Q rows requested above arrive with them)
+    asm volatile("s_waitcnt vmcnt(0)"
+                 : "+v"(first_slots[0]), "+v"(first_slots[1]), "+v"(first_slots[2]), "+v"(first_slots[3]),
+                   "+v"(sl)
+                 :
+                 : "memory");
 #pragma unroll
     for (int x = 0; x < 4; ++x) {
-      slot_load(k_lo + x * kHalf, sl);
-      wait_vm_and_slots(std::integral_constant<int, 0>{}, sl);
 #pragma unroll
       for (int i = 0; i < kUPW; ++i) {
-        k_off[i] = lane_offset(sl[i], k_row_bytes);
-        v_off[x & 1][i] = lane_offset(sl[i], v_row_bytes);
+        k_off[i] = lane_offset(first_slots[x][i], k_row_bytes);
+        v_off[x & 1][i] = lane_offset(first_slots[x][i], v_row_bytes);
       }
 #pragma unroll
       for (int n = (x < 2 ? 0 : kUPW); n < kMovesPerStep; ++n)
         move(n, x * kKStage, kVBase + x * kVStage, v_off[x & 1]);
       // the V offsets of halves 2 and 3 stay in v_off[0], v_off[1] for the moves of steps 0 and 1
     }
-    // everything but K of half 3 has to have landed; the ids for the K move of step 0 ride along
-    slot_load(k_lo + 4 * kHalf, sl);
-    wait_vm_and_slots(std::integral_constant<int, 0>{}, sl);
+    // everything but K of half 3 has to have landed
+    wait_vm_at_most<kUPW>();
     __syncthreads();
 
     f32x16_t sa = zero16, sb;
