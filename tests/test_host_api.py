@@ -188,8 +188,10 @@ def test_mha_kv_cache_and_backend_host_logic():
     assert torch.count_nonzero(pool.v_cache(0)) == 0
     with pytest.raises(AssertionError, match="out_loc must be int32"):
         pool.store_kv(_t((2, 2, 128)), _t((2, 2, 128)), torch.zeros(2, dtype=torch.int64), 0)
-    with pytest.raises(ValueError, match="store_kv shape mismatch"):
+    with pytest.raises(ValueError, match="3 slot ids for k of shape"):  # mha_pool.py:42-46
         pool.store_kv(_t((2, 2, 128)), _t((2, 2, 128)), _i(3), 0)
+    assert pool.pool_shape == (9, 2, 128) and pool.nbytes == 2 * 3 * 9 * 2 * 128 * 2
+    assert pool.k_cache(1).is_contiguous() and pool.k_cache(1).stride(0) == 2 * 128
 
     # closed forms of backend.py:299-307
     assert _build_indptr([3, 0, 5]).tolist() == [0, 3, 3, 8]
