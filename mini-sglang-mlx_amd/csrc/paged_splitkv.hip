@@ -583,7 +583,9 @@ int launch_dn(const SplitKvParams& p, int waves, hipStream_t stream) {
 // How a shape's column tiles map onto waves: tiles per wave and waves per kv head.
 struct ColSplit { int nct_wave; int col_waves; };
 ColSplit col_split(int nct, int64_t head_dim) {
-  if (head_dim != 128) return ColSplit{1, nct};  // two tiles at head dim 256 would spill
+  // head dim 256: one tile per wave (two would spill); three tiles take four waves, the last
+  // of which finds no valid column (workgroups come in 1, 2, 4 or 8 waves)
+  if (head_dim != 128) return ColSplit{1, nct == 3 ? 4 : nct};
   return nct <= 2 ? ColSplit{nct, 1} : ColSplit{2, 2};
 }
 

@@ -2,6 +2,7 @@
 head sizes, page sizes, ragged lengths (empty requests, single tokens, lengths around the 16-,
 32- and 64-key tile edges), every mask, with and without a store first.  The fixed cases of the
 other modules aim at known edges; this one looks for the ones nobody thought of."""
+import os
 import random
 
 import pytest
@@ -13,6 +14,8 @@ from mini_sglang_amd.workloads import build_workload
 
 pytestmark = pytest.mark.gpu
 
+# more seeds on request: MSGL_FUZZ_SCALE=10 runs ten times as many cases
+_SCALE = max(1, int(os.environ.get("MSGL_FUZZ_SCALE", "1")))
 HEADS = [(1, 1), (2, 1), (4, 4), (6, 3), (8, 2), (8, 8), (12, 4), (16, 1), (16, 8), (20, 4), (32, 8)]
 EDGES = [0, 1, 2, 15, 16, 17, 31, 32, 33, 47, 63, 64, 65, 95, 96, 97, 127, 128, 129, 255, 257]
 
@@ -21,7 +24,7 @@ def _length(rng, hi):
     return rng.choice(EDGES) if rng.random() < 0.5 else rng.randrange(0, hi)
 
 
-@pytest.mark.parametrize("seed", range(40))
+@pytest.mark.parametrize("seed", range(80 * _SCALE))
 def test_random_prefill_shapes(gpu, seed):
     rng = random.Random(1000 + seed)
     n_q, n_kv = rng.choice(HEADS)
@@ -58,7 +61,7 @@ def test_random_prefill_shapes(gpu, seed):
         assert torch.equal(g.v_cache.cpu().view(torch.int16), ref.v_cache.view(torch.int16)), what
 
 
-@pytest.mark.parametrize("seed", range(25))
+@pytest.mark.parametrize("seed", range(40 * _SCALE))
 def test_random_decode_shapes(gpu, seed):
     rng = random.Random(2000 + seed)
     n_q, n_kv = rng.choice([h for h in HEADS if h[0] // h[1] <= 16])

@@ -189,6 +189,19 @@ def test_head_dim_256_tile_kernel_unusual_scales_and_magnitudes(gpu, scale):
     _check(big, gpu, "head_dim 256 large magnitude")
 
 
+@pytest.mark.parametrize("head_dim", [128, 256])
+@pytest.mark.parametrize("n_q,n_kv,q_len", [(8, 8, 36), (8, 8, 48), (8, 4, 20), (4, 4, 64), (6, 2, 11),
+                                            (8, 8, 17), (16, 1, 3)])
+def test_splitk_route_every_column_tile_count(gpu, head_dim, n_q, n_kv, q_len):
+    # q_len * group = 36, 48, 40, 64, 33, 17, 48 columns: two, three and four tiles of 16, the
+    # three-tile ones with an idle fourth wave per kv head at head_dim 256
+    wl = build_workload("t", "prefill", seed=390 + q_len, n_q=n_q, n_kv=n_kv, head_dim=head_dim,
+                        kv_lens=[q_len + 32, 500 + q_len, q_len], extend_lens=[q_len] * 3,
+                        pool_factor=1.2, store_new=True, sliding_window_size=0)
+    _check(wl, gpu, f"split-K columns d={head_dim} heads={n_q}/{n_kv} q_len={q_len}")
+    _check(wl.with_mask(is_cross_attention=False, sliding_window_size=2), gpu, "same, window 2")
+
+
 @pytest.mark.parametrize("scale", [0.0, -0.3, 1.5, 0.01])
 def test_unusual_softmax_scales_on_both_routes(gpu, tile_variant, scale):
     # zero (uniform weights), negative (the smallest score wins), large (peaky rows: the running
