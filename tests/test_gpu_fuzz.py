@@ -79,3 +79,74 @@ def test_random_decode_shapes(gpu, seed):
     for b, l in enumerate(kv):
         if l == 0:
             assert torch.count_nonzero(got[b]) == 0, what
+
+
+@pytest.mark.parametrize("seed", range(30 * _SCALE))
+def test_random_metadata_builds(gpu, seed):
+    import numpy as np
+
+    from oracle import metadata_oracle as mo
+    from test_gpu_metadata import _case, _run
+
+    rng = np.random.default_rng(3000 + seed)
+    batch = int(rng.choice([1, 2, 3, 17, 63, 64, 65, 200, 1000]))
+    rows = int(rng.integers(1, 70))
+    max_seq = int(rng.choice([1, 2, 31, 32, 33, 255, 257, 1000, 4100]))
+    table, trows, kv, ext = _case(rng, batch, rows, max_seq, zero_frac=float(rng.choice([0.0, 0.1, 0.6])))
+    decode = rng.random() < 0.3
+    print(f"fuzz metadata seed={seed} batch={batch} rows={rows} max_seq={max_seq} decode={decode}", flush=True)
+    if decode:
+        kv = np.maximum(kv, 1)
+        got = _run(gpu, table, trows, kv, None, total_kv=int(kv.sum()))
+        want = mo.build_decode_metadata(table, trows, kv)
+        keys = ("kv_indptr", "kv_indices", "num_kv_splits", "positions")
+    else:
+        got = _run(gpu, table, trows, kv, ext, total_kv=int(kv.sum()), total_q=int(ext.sum()))
+        want = mo.build_prefill_metadata(table, trows, kv, ext)
+        keys = ("kv_indptr", "kv_indices", "qo_indptr", "prefix_lens", "positions", "num_kv_splits")
+    for k in keys:
+        np.testing.assert_array_equal(got[k], want[k], err_msg=f"{k} seed={seed}")
+
+
+@pytest.mark.parametrize("seed", range(20 * _SCALE))
+def test_random_norm_rope_store_shapes(gpu, seed):
+    from test_gpu_qk_norm_rope import _run_case
+
+    rng = random.Random(4000 + seed)
+    n_q, n_kv = rng.choice(HEADS)
+    d = rng.choice([128, 128, 256])
+    L = rng.choice([1, 2, 7, 63, 64, 65, 300, 1025])
+    _run_case(gpu, L, n_q, n_kv, d, slots=L + rng.randrange(0, 50), max_pos=rng.choice([0, 100, 9000, 100000]),
+              base=rng.choice([1e4, 1e6]), seed=seed, fused_view=rng.random() < 0.4)
+
+
+@pytest.mark.parametrize("seed", range(16 * _SCALE))
+def test_random_gdn_state_shapes(gpu, seed):
+    import numpy as np
+
+    from oracle import gdn_state_oracle as go
+    from test_gpu_gdn_state import _check, _gpu, _inputs
+
+    rng = np.random.default_rng(5000 + seed)
+    hk = int(rng.choice([1, 2, 4, 16]))
+    hv = hk * int(rng.choice([1, 2, 3]))
+    single = rng.random() < 0.4
+    if single:
+        batch = int(rng.choice([1, 3, 8, 33, 100]))
+        lengths = [1] * batch
+    else:
+        batch = int(rng.integers(1, 7))
+        lengths = [int(rng.choice([0, 1, 2, 9, 40, 130])) for _ in range(batch)]
+        if sum(lengths) == 0:
+            lengths[0] = 5
+    total = sum(lengths)
+    d, state = _inputs(rng, total, hk, hv, batch + 4)
+    slots = rng.permutation(batch + 4)[:batch]
+    indptr = np.concatenate([[0], np.cumsum(lengths)])
+    print(f"fuzz gdn seed={seed} hk={hk} hv={hv} single={single} lengths={lengths[:8]}", flush=True)
+    got_y, got_st = _gpu(gpu, d, state, slots, indptr, single)
+    want_y, want_st = go.gdn_state_inplace(d["q"], d["k"], d["v"], d["g"], d["beta"], state, slots,
+                                           None if single else indptr, single_token_mode=single)
+    _check(got_y, got_st, want_y, want_st, f"fuzz gdn seed={seed}")
+    other = np.setdiff1d(np.arange(state.shape[0]), slots)
+    np.testing.assert_array_equal(got_st[other], state[other])

@@ -51,13 +51,20 @@ def _run_case(gpu, L, n_q, n_kv, d, slots, max_pos, base, seed, fused_view=False
         h = want.shape[-1] // 2
         pair = np.hypot(want[..., :h], want[..., h:])  # an angle error moves a value by angle * pair norm
         pair = np.concatenate([pair, pair], axis=-1)
-        step = 2.0 ** -7 * np.maximum(np.abs(want), 2.0 ** -6) + 2e-7 * max_pos * pair
+        # (a value is x cos - y sin of a pair of norm `pair`: an intermediate rounding of x or y
+        # moves it by a step of THEIR size, however small the difference comes out)
+        step = 2.0 ** -7 * np.maximum(np.maximum(np.abs(want), pair), 2.0 ** -6) + 2e-7 * max_pos * pair
         # An intermediate rounding (normalised value, weighted value) that sits on a tie can fall
         # the other way with float32 statistics; that moves a result by up to two more steps
         # and is rare.
         assert np.all(diff <= 3 * step), (name, float(diff.max()), float((diff / step).max()))
         assert np.mean(diff > step) < 5e-3, (name, float(np.mean(diff > step)))
-        assert diff.max() <= 2e-2 * max(1.0, np.abs(want).max() / 4) and diff.mean() <= 2e-3, name
+        # the path's stated tolerance, plus what float32 angles cost at this position range
+        # (pos * inv_freq carries 2^-24 of pos radians: 6e-3 rad at position 100000)
+        angle_slack = 2e-7 * max_pos * float(pair.max())
+        # (2e-2 on unit-scale values; one bf16 step of the largest value where that is more)
+        assert diff.max() <= max(2e-2, 2.0 ** -7 * float(np.abs(want).max())) + angle_slack, name
+        assert diff.mean() <= 2e-3 + 2e-7 * max_pos * float(pair.mean()), name
     return got_q
 
 
