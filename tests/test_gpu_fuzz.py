@@ -150,3 +150,89 @@ def test_random_gdn_state_shapes(gpu, seed):
     _check(got_y, got_st, want_y, want_st, f"fuzz gdn seed={seed}")
     other = np.setdiff1d(np.arange(state.shape[0]), slots)
     np.testing.assert_array_equal(got_st[other], state[other])
+
+
+MORE_HEADS = HEADS + [(7, 1), (10, 2), (32, 1), (48, 2), (40, 8), (64, 8), (3, 3)]
+
+
+def _strided(pool, pad_elems):
+    """The same pool values in a buffer whose slots are `pad_elems` further apart."""
+    slots, n_kv, d = pool.shape
+    buf = torch.zeros((slots, n_kv * d + pad_elems), dtype=pool.dtype, device=pool.device)
+    view = buf[:, : n_kv * d].view(slots, n_kv, d)
+    view.copy_(pool)
+    return view
+
+
+@pytest.mark.parametrize("seed", range(40 * _SCALE))
+def test_random_prefill_strides_heads_and_query_caps(gpu, seed):
+    """More of the argument space: odd head counts and large groups, pools with padded slots,
+    a `max_len_extend` below the longest extend (rows past it are not computed, as in the
+    reference's grid, paged_prefill_attention.cpp:152-159), a caller-owned stream."""
+    import dataclasses
+
+    from mini_sglang_amd_kernel import paged_prefill_attention, store_kv_cache
+
+    rng = random.Random(6000 + seed)
+    n_q, n_kv = rng.choice(MORE_HEADS)
+    d = rng.choice([128, 256])
+    batch = rng.randrange(1, 5)
+    ext = [rng.choice([1, 2, 5, 16, 17, 40, 70, 129, 200]) for _ in range(batch)]
+    kv = [e + (_length(rng, 400) if rng.random() < 0.8 else 0) for e in ext]
+    wl = build_workload("fuzz", "prefill", seed=seed, n_q=n_q, n_kv=n_kv, head_dim=d,
+                        page_size=rng.choice([1, 16]), kv_lens=kv, extend_lens=ext, pool_factor=1.3,
+                        store_new=True, is_cross_attention=rng.random() < 0.3,
+                        sliding_window_size=rng.choice([0, 0, 3, 50, 300]))
+    cap = max(ext) if rng.random() < 0.6 else rng.randrange(1, max(ext) + 1)
+    wl = dataclasses.replace(wl, max_len_extend=cap)
+    pad = rng.choice([0, 8, 64, 1000 * 8])
+    what = (f"fuzz prefill+ seed={seed} heads={n_q}/{n_kv} d={d} ext={ext} kv={kv} cap={cap} pad={pad} "
+            f"cross={wl.is_cross_attention} W={wl.sliding_window_size}")
+    print(what, flush=True)
+    g = wl.to(gpu)
+    kc, vc = _strided(g.k_cache, pad), _strided(g.v_cache, pad)
+    side = torch.cuda.Stream(device=gpu)
+    side.wait_stream(torch.cuda.current_stream(gpu))
+    with torch.cuda.stream(side):
+        store_kv_cache(kc, vc, g.out_loc, g.new_k, g.new_v, stream=side)
+        got = paged_prefill_attention(g.q, kc, vc, g.qo_indptr, g.kv_indptr, g.kv_indices,
+                                      g.prefix_lens, g.sm_scale, cap,
+                                      is_cross_attention=g.is_cross_attention,
+                                      sliding_window_size=g.sliding_window_size, stream=side)
+    side.synchronize()
+    want, ref = run_oracle(wl)
+    qo = wl.qo_indptr.tolist()
+    rows = torch.cat([torch.arange(qo[b], qo[b] + min(ext[b], cap)) for b in range(batch)])
+    assert_close_bf16(got.cpu()[rows], want[rows], what)
+    assert torch.equal(kc.cpu().view(torch.int16), ref.k_cache.view(torch.int16)), what
+    assert torch.equal(vc.cpu().view(torch.int16), ref.v_cache.view(torch.int16)), what
+
+
+@pytest.mark.parametrize("seed", range(30 * _SCALE))
+def test_random_decode_half_precision_and_strides(gpu, seed):
+    from mini_sglang_amd_kernel import paged_decode_attention
+    from test_gpu_decode import _as_half
+
+    rng = random.Random(7000 + seed)
+    n_q, n_kv = rng.choice([h for h in MORE_HEADS if h[0] // h[1] <= 16])
+    d = rng.choice([128, 256])
+    batch = rng.randrange(1, 20)
+    kv = [_length(rng, 1500) for _ in range(batch)]
+    wl = build_workload("fuzz", "decode", seed=seed, n_q=n_q, n_kv=n_kv, head_dim=d,
+                        page_size=rng.choice([1, 16]), kv_lens=kv, pool_factor=1.2)
+    half = rng.random() < 0.5
+    pad = rng.choice([0, 8, 264])
+    what = f"fuzz decode+ seed={seed} heads={n_q}/{n_kv} d={d} batch={batch} half={half} pad={pad}"
+    print(what, flush=True)
+    as_bf16, as_half = _as_half(wl)
+    src = (as_half if half else as_bf16).to(gpu)
+    got = paged_decode_attention(src.q, _strided(src.k_cache, pad), _strided(src.v_cache, pad),
+                                 src.kv_indptr, src.kv_indices, src.num_kv_splits, src.sm_scale,
+                                 src.max_kv_splits)
+    torch.cuda.synchronize()
+    assert got.dtype == (torch.float16 if half else torch.bfloat16)
+    want, _ = run_oracle(as_bf16)
+    if half:
+        assert_close_bf16(got, want, what, max_tol=5e-3, mean_tol=4e-4)
+    else:
+        assert_close_bf16(got, want, what)
