@@ -82,6 +82,7 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
   // decreasing kv length (longest-processing-time-first: the dispatcher hands out blocks
   // in id order, so long requests start first and short ones fill the tail); each block
   // finds "the request of rank r" itself from kv_indptr, the host never sees the lengths.
+  // Beyond kRankedBatch requests the order is the batch order.
   const int xcd = blockIdx.x & 7;
   const int seq = blockIdx.x >> 3;
   const int pair = (seq / p.n_qblk) * 8 + xcd;
@@ -90,14 +91,18 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
   const int want_rank = pair / p.n_kv;
   const int kvh = pair - want_rank * p.n_kv;
   __shared__ int ranked_request;
-  for (int i = tid; i < p.batch; i += NW * 64) {
-    const int len_i = p.kv_indptr[i + 1] - p.kv_indptr[i];
-    int rank = 0;
-    for (int j = 0; j < p.batch; ++j) {
-      const int len_j = p.kv_indptr[j + 1] - p.kv_indptr[j];
-      rank += (len_j > len_i) || (len_j == len_i && j < i);
+  if (p.batch <= kRankedBatch) {
+    for (int i = tid; i < p.batch; i += NW * 64) {
+      const int len_i = p.kv_indptr[i + 1] - p.kv_indptr[i];
+      int rank = 0;
+      for (int j = 0; j < p.batch; ++j) {
+        const int len_j = p.kv_indptr[j + 1] - p.kv_indptr[j];
+        rank += (len_j > len_i) || (len_j == len_i && j < i);
+      }
+      if (rank == want_rank) ranked_request = i;
     }
-    if (rank == want_rank) ranked_request = i;
+  } else if (tid == 0) {
+    ranked_request = want_rank;  // many requests balance by their number: batch order
   }
   __syncthreads();
   const int b = ranked_request;

@@ -78,14 +78,18 @@ __global__ __launch_bounds__(kNW * 64) void prefill_tile256_kernel(PrefillParams
   const int want_rank = pair / p.n_kv;
   const int kvh = pair - want_rank * p.n_kv;
   __shared__ int ranked_request;
-  for (int i = tid; i < p.batch; i += kNW * 64) {
-    const int len_i = p.kv_indptr[i + 1] - p.kv_indptr[i];
-    int rank = 0;
-    for (int j = 0; j < p.batch; ++j) {
-      const int len_j = p.kv_indptr[j + 1] - p.kv_indptr[j];
-      rank += (len_j > len_i) || (len_j == len_i && j < i);
+  if (p.batch <= kRankedBatch) {
+    for (int i = tid; i < p.batch; i += kNW * 64) {
+      const int len_i = p.kv_indptr[i + 1] - p.kv_indptr[i];
+      int rank = 0;
+      for (int j = 0; j < p.batch; ++j) {
+        const int len_j = p.kv_indptr[j + 1] - p.kv_indptr[j];
+        rank += (len_j > len_i) || (len_j == len_i && j < i);
+      }
+      if (rank == want_rank) ranked_request = i;
     }
-    if (rank == want_rank) ranked_request = i;
+  } else if (tid == 0) {
+    ranked_request = want_rank;  // many requests balance by their number: batch order
   }
   __syncthreads();
   const int b = __builtin_amdgcn_readfirstlane(ranked_request);

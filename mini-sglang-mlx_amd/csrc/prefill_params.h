@@ -27,6 +27,10 @@ constexpr int kBN = 64;  // keys per tile
 // A stale row max is kept until the new one exceeds it by this much (base-2 exponent):
 // P stays below 2^kLazy, far inside bf16 / fp32 range, and O is rescaled rarely.
 constexpr float kLazy = 8.0f;
+// Requests are processed longest first only up to this batch size: every workgroup ranks the
+// requests itself (batch^2 comparisons spread over its threads), which stops paying when there
+// are many of them.
+constexpr int kRankedBatch = 128;
 constexpr int kPrefillBlockRows = 256;      // rows per workgroup, head_dim 128
 constexpr int kPrefillBlockRows256 = 128;   // head_dim 256
 

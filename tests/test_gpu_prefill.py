@@ -202,6 +202,20 @@ def test_splitk_route_every_column_tile_count(gpu, head_dim, n_q, n_kv, q_len):
     _check(wl.with_mask(is_cross_attention=False, sliding_window_size=2), gpu, "same, window 2")
 
 
+@pytest.mark.parametrize("head_dim", [128, 256])
+def test_tile_route_many_requests(gpu, head_dim):
+    # more requests than the kernels rank by length (they then go in batch order): 150 and 129
+    # ragged extends, with one batch exactly at the limit
+    for batch in (128, 129, 150):
+        g = torch.Generator().manual_seed(batch)
+        ext = torch.randint(17, 90, (batch,), generator=g).tolist()
+        pre = torch.randint(0, 60, (batch,), generator=g).tolist()
+        wl = build_workload("t", "prefill", seed=500 + batch, n_q=8, n_kv=2, head_dim=head_dim,
+                            kv_lens=[p + e for p, e in zip(pre, ext)], extend_lens=ext,
+                            pool_factor=1.1, store_new=True)
+        _check(wl, gpu, f"tile route d={head_dim} batch={batch}")
+
+
 @pytest.mark.parametrize("scale", [0.0, -0.3, 1.5, 0.01])
 def test_unusual_softmax_scales_on_both_routes(gpu, tile_variant, scale):
     # zero (uniform weights), negative (the smallest score wins), large (peaky rows: the running
