@@ -119,7 +119,11 @@ MSGL_API int msgl_paged_decode_attention(const void* q, const void* k_cache, con
                                 float sm_scale, int32_t max_kv_splits,
                                 int32_t dtype, void* stream);
 
-/* Workspace (bytes) that msgl_paged_prefill_attention needs for these sizes. */
+/*
+ * Workspace (bytes) that msgl_paged_prefill_attention needs for these sizes: the partials of the
+ * split-K route, or those of the tile kernels when the launch is too small to fill the chip and
+ * the keys of each query block are shared out over several workgroups; 0 otherwise.
+ */
 MSGL_API size_t msgl_paged_prefill_workspace_bytes(int64_t batch, int64_t total_q, int64_t total_kv,
                                           int64_t num_q_heads, int64_t num_kv_heads,
                                           int64_t head_dim, int64_t max_len_extend);
@@ -137,7 +141,10 @@ MSGL_API size_t msgl_paged_prefill_workspace_bytes(int64_t batch, int64_t total_
  * for their first max_len_extend queries, as in the reference's grid
  * (paged_prefill_attention.cpp:152-159).  Short query blocks (speculative verify,
  * draft proposal) are routed to the bandwidth-bound split-K kernel, long ones to
- * the MFMA tile kernel of their head_dim; same arguments, same result.
+ * the MFMA tile kernel of their head_dim; same arguments, same result.  A launch of the tile
+ * kernels with fewer query blocks than compute units (one long request, a short extend) shares
+ * the keys of every block out over up to 32 workgroups and merges their fp32 partials by
+ * log-sum-exp in a second kernel.
  */
 MSGL_API int msgl_paged_prefill_attention(const void* q, const void* k_cache, const void* v_cache,
                                  const int32_t* qo_indptr, const int32_t* kv_indptr,
@@ -237,6 +244,8 @@ MSGL_API int msgl_gdn_state_inplace(const void* q, const void* k, const void* v,
  *                            (0 restores the default, 4)
  *   MSGL_TUNE_GDN_ROWS       state rows per 16-lane group of the gdn_state kernel: 1, 2, 4
  *                            (0: chosen from the problem size)
+ *   MSGL_TUNE_PREFILL_KEY_SPLITS  workgroups that share the keys of one query block of the MFMA
+ *                            tile kernels (1: never split, up to 32; 0: chosen from the sizes)
  */
 #define MSGL_TUNE_SEGMENTS 0
 #define MSGL_TUNE_MIN_SEGMENT 1
@@ -244,6 +253,7 @@ MSGL_API int msgl_gdn_state_inplace(const void* q, const void* k, const void* v,
 #define MSGL_TUNE_PREFILL_VARIANT 3
 #define MSGL_TUNE_SPLITKV_WAVES 4
 #define MSGL_TUNE_GDN_ROWS 5
+#define MSGL_TUNE_PREFILL_KEY_SPLITS 6
 MSGL_API int msgl_set_tuning(int32_t knob, int64_t value);
 
 #ifdef __cplusplus

@@ -7,10 +7,12 @@
 #include <algorithm>
 
 #include "msgl_internal.h"
+#include "prefill_params.h"
 
 namespace {
 
 std::atomic<int64_t> g_tune[3] = {{0}, {0}, {0}};
+std::atomic<int64_t> g_key_splits{0};
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
@@ -86,6 +88,10 @@ int msgl_set_tuning(int32_t knob, int64_t value) {
   }
   if (knob == MSGL_TUNE_PREFILL_VARIANT) {
     msgl::set_tile_variant((int)value);
+    return MSGL_OK;
+  }
+  if (knob == MSGL_TUNE_PREFILL_KEY_SPLITS) {
+    g_key_splits.store(value < 0 ? 0 : value);
     return MSGL_OK;
   }
   if (knob < 0 || knob > 2) return MSGL_ERR_SHAPE;
@@ -186,13 +192,18 @@ static int32_t chunk_queries(int64_t group) {
 size_t msgl_paged_prefill_workspace_bytes(int64_t batch, int64_t total_q, int64_t total_kv,
                                           int64_t num_q_heads, int64_t num_kv_heads,
                                           int64_t head_dim, int64_t max_len_extend) {
-  (void)total_q;
-  if (batch <= 0 || total_kv < 0 || num_q_heads <= 0 || num_kv_heads <= 0 ||
+  if (batch <= 0 || total_q < 0 || total_kv < 0 || num_q_heads <= 0 || num_kv_heads <= 0 ||
       num_q_heads % num_kv_heads != 0)
     return 0;
   const int64_t group = num_q_heads / num_kv_heads;
   if (!use_splitkv_route(group, max_len_extend)) {
-    if (!use_chunked_route(head_dim, group)) return 0;
+    if (!use_chunked_route(head_dim, group)) {
+      // tile kernels: partials of a key split, if this launch would use one (a sliding window,
+      // unknown here, can only lower the count)
+      const int k = msgl::prefill_key_splits(batch, total_kv, num_kv_heads, group, max_len_extend, 0,
+                                             msgl::prefill_block_rows(head_dim), g_key_splits.load());
+      return msgl::prefill_split_workspace_bytes(total_q, num_q_heads, head_dim, k);
+    }
     const int32_t qc = chunk_queries(group);
     return msgl::splitkv_workspace_bytes(batch, num_q_heads, num_kv_heads, head_dim, qc,
                                          segments(total_kv, num_kv_heads, head_dim, group * qc));
@@ -287,6 +298,14 @@ int msgl_paged_prefill_attention(const void* q, const void* k_cache, const void*
   a.max_len_extend = max_len_extend;
   a.is_cross = is_cross_attention ? 1 : 0;
   a.window = sliding_window_size;
+  a.key_splits = msgl::prefill_key_splits(batch, total_kv, num_kv_heads, group, max_len_extend,
+                                          sliding_window_size, msgl::prefill_block_rows(head_dim),
+                                          g_key_splits.load());
+  if (a.key_splits > 1) {
+    const size_t need = msgl::prefill_split_workspace_bytes(total_q, num_q_heads, head_dim, a.key_splits);
+    if (!workspace || workspace_bytes < need || !aligned16(workspace)) return MSGL_ERR_WORKSPACE;
+    a.workspace = workspace;
+  }
   return head_dim == 256 ? msgl::launch_prefill_tile256(a, s) : msgl::launch_prefill_tile(a, s);
 }
 

@@ -66,6 +66,10 @@ struct PrefillArgs {
   float sm_scale;
   int32_t max_len_extend;
   int32_t is_cross, window;
+  // key splits (1: none); above 1, `workspace` holds
+  // key_splits * total_q * n_q * (head_dim + 1) floats
+  int32_t key_splits;
+  void* workspace;
 };
 int launch_prefill_tile(const PrefillArgs& a, hipStream_t stream);     // head_dim 128
 // ---- paged_prefill_d256.hip ----------------------------------------------------------

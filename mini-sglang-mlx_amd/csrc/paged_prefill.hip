@@ -76,17 +76,19 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
   const int h = lane >> 5;
   const int c32 = lane & 31;
 
-  // ---- block -> (request, kv head, q block).  Consecutive block ids go to different
-  // XCDs; the q blocks of one (request, kv head) share an XCD (and its L2) and are
-  // issued back to back, heaviest (latest rows) first.  Requests are taken in order of
+  // ---- block -> (request, kv head, key split, q block).  Consecutive block ids go to
+  // different XCDs; the q blocks of one (request, kv head, key split) read the same keys,
+  // share an XCD (and its L2) and are issued back to back, heaviest (latest rows) first.  Requests are taken in order of
   // decreasing kv length (longest-processing-time-first: the dispatcher hands out blocks
   // in id order, so long requests start first and short ones fill the tail); each block
   // finds "the request of rank r" itself from kv_indptr, the host never sees the lengths.
   // Beyond kRankedBatch requests the order is the batch order.
   const int xcd = blockIdx.x & 7;
   const int seq = blockIdx.x >> 3;
-  const int pair = (seq / p.n_qblk) * 8 + xcd;
-  if (pair >= p.n_pairs) return;
+  const int unit = (seq / p.n_qblk) * 8 + xcd;  // (request, kv head, key split)
+  if (unit >= p.n_pairs * p.n_ksplit) return;
+  const int pair = unit / p.n_ksplit;
+  const int split = unit - pair * p.n_ksplit;
   const int qblk = p.n_qblk - 1 - (seq % p.n_qblk);
   const int want_rank = pair / p.n_kv;
   const int kvh = pair - want_rank * p.n_kv;
@@ -122,6 +124,14 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
   int k_lo = (p.window > 0) ? max(0, prefix + qi_lo - p.window + 1) : 0;
   k_lo &= ~(kBN - 1);
   if (k_hi < k_lo) k_hi = k_lo;
+  // key split `split` of n_ksplit: a whole number of tiles each, the last takes the ragged end;
+  // shares past the end are empty (they still leave their "nothing seen" partial)
+  if (p.n_ksplit > 1) {
+    const int all_tiles = (k_hi - k_lo + kBN - 1) / kBN;
+    const int share = (all_tiles + p.n_ksplit - 1) / p.n_ksplit * kBN;
+    k_lo = min(k_lo + split * share, k_hi);
+    k_hi = min(k_hi, k_lo + share);
+  }
   const int n_tiles = (k_hi - k_lo + kBN - 1) / kBN;
 
   // ---- per-lane rows: Q operand, visibility bounds ---------------------------------
@@ -143,7 +153,8 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
     }
     const int qpos = prefix + qi;
     int lo = (p.window > 0) ? qpos - p.window + 1 : 0;
-    int hi = p.is_cross ? kn - 1 : min(qpos, kn - 1);
+    // k_hi - 1 only binds under a key split: the pipeline looks one half tile past its share
+    int hi = min(p.is_cross ? kn - 1 : min(qpos, kn - 1), k_hi - 1);
     if (valid) {
       w_lo_max = max(w_lo_max, lo);
       w_hi_min = min(w_hi_min, hi);
@@ -547,8 +558,34 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
 #endif
   }
 
-  // ---- epilogue: normalise, transpose through LDS, store whole rows ---------------------
   // accumulator i of O^T tile dt is dim 32dt + 8(i/4) + 4h + i%4 of query row c32
+  if (p.n_ksplit > 1) {
+    // ---- key split: normalised fp32 partial and log-sum-exp (base 2) per row, from registers
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      float l = l_run[rt];
+      l += __shfl_xor(l, 32, kWave);
+      const float inv = (l > 0.f) ? 1.0f / l : 0.f;
+      const int row = row0 + (w * RT + rt) * 32 + c32;
+      if (row < rows_total) {
+        const int qi = row / p.group;
+        const int hh = row - qi * p.group;
+        const int64_t at = (int64_t)split * p.part_rows + (int64_t)(q_start + qi) * p.n_q + kvh * p.group + hh;
+        if (h == 0) p.part_lse[at] = (l > 0.f) ? m_run[rt] + __log2f(l) : kNegInf;
+        float* dst = p.part_o + at * D + 4 * h;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+          for (int a = 0; a < 4; ++a) {
+            f32x4_t v = {oacc[dt][rt][4 * a] * inv, oacc[dt][rt][4 * a + 1] * inv,
+                         oacc[dt][rt][4 * a + 2] * inv, oacc[dt][rt][4 * a + 3] * inv};
+            *reinterpret_cast<f32x4_t*>(dst + 32 * dt + 8 * a) = v;
+          }
+      }
+    }
+    return;
+  }
+  // ---- epilogue: normalise, transpose through LDS, store whole rows ---------------------
   unsigned char* os = smem;
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
@@ -582,7 +619,65 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
   }
 }
 
+
+// ---- merge of a key-split launch: one 32-lane group per (token, q head) row -----------------
+template <int D>
+__global__ __launch_bounds__(256) void prefill_merge_kernel(const float* __restrict__ part_o,
+                                                            const float* __restrict__ part_lse,
+                                                            const int32_t* __restrict__ qo_indptr,
+                                                            uint16_t* __restrict__ out, int64_t part_rows,
+                                                            int n_q, int n_ksplit, int max_len_extend) {
+  constexpr int V = D / 32;  // dims per lane
+  const int b = blockIdx.y;
+  const int q_start = qo_indptr[b];
+  const int q_len = min(qo_indptr[b + 1] - q_start, max_len_extend);
+  const int64_t r = (int64_t)blockIdx.x * 8 + (threadIdx.x >> 5);  // row of the request, token-major
+  if (r >= (int64_t)q_len * n_q) return;
+  const int64_t row = (int64_t)q_start * n_q + r;
+  const int c = threadIdx.x & 31;
+  float top = kNegInf;
+  for (int s = 0; s < n_ksplit; ++s) top = fmaxf(top, part_lse[s * part_rows + row]);
+  float acc[V];
+#pragma unroll
+  for (int i = 0; i < V; ++i) acc[i] = 0.f;
+  float total = 0.f;
+  for (int s = 0; s < n_ksplit; ++s) {
+    const float lse = part_lse[s * part_rows + row];
+    if (lse == kNegInf) continue;  // that share saw no key of this row
+    const float wgt = exp2f(lse - top);
+    total += wgt;
+    const float* src = part_o + (s * part_rows + row) * D + c * V;
+#pragma unroll
+    for (int i = 0; i < V; i += 4) {
+      const f32x4_t x = *reinterpret_cast<const f32x4_t*>(src + i);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc[i + e] += wgt * x[e];
+    }
+  }
+  const float inv = (total > 0.f) ? 1.0f / total : 0.f;
+  uint16_t* dst = out + row * D + c * V;
+#pragma unroll
+  for (int i = 0; i < V; i += 4) {
+    u32x2_t wv;
+    wv[0] = pack_bf16x2(acc[i] * inv, acc[i + 1] * inv);
+    wv[1] = pack_bf16x2(acc[i + 2] * inv, acc[i + 3] * inv);
+    *reinterpret_cast<u32x2_t*>(dst + i) = wv;
+  }
+}
+
 }  // namespace
+
+int launch_prefill_merge(const PrefillParams& p, int head_dim, hipStream_t stream) {
+  const int64_t rows = (int64_t)p.max_len_extend * p.n_q;
+  const dim3 grid((unsigned)((rows + 7) / 8), (unsigned)p.batch);
+  if (head_dim == 256)
+    hipLaunchKernelGGL((prefill_merge_kernel<256>), grid, dim3(256), 0, stream, p.part_o, p.part_lse,
+                       p.qo_indptr, p.out, p.part_rows, p.n_q, p.n_ksplit, p.max_len_extend);
+  else
+    hipLaunchKernelGGL((prefill_merge_kernel<128>), grid, dim3(256), 0, stream, p.part_o, p.part_lse,
+                       p.qo_indptr, p.out, p.part_rows, p.n_q, p.n_ksplit, p.max_len_extend);
+  return check_launch();
+}
 
 #ifdef MSGL_PROFILE_PHASES
 static long long* g_prof_buf = nullptr;
@@ -613,7 +708,9 @@ int launch_prefill_tile(const PrefillArgs& a, hipStream_t stream) {
     if (wide) hipLaunchKernelGGL((prefill_tile_kernel<128, 1, 8, true>), grid, dim3(512), 0, stream, p);
     else hipLaunchKernelGGL((prefill_tile_kernel<128, 1, 8, false>), grid, dim3(512), 0, stream, p);
   }
-  return check_launch();
+  const int launched = check_launch();
+  if (launched != MSGL_OK || p.n_ksplit == 1) return launched;
+  return launch_prefill_merge(p, 128, stream);
 }
 
 }  // namespace msgl

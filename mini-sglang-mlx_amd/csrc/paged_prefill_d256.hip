@@ -67,13 +67,16 @@ __global__ __launch_bounds__(kNW * 64) void prefill_tile256_kernel(PrefillParams
   const int h = lane >> 5;
   const int c32 = lane & 31;
 
-  // ---- block -> (request, kv head, q block): consecutive block ids go to different XCDs, the
-  // q blocks of one (request, kv head) share an XCD and run heaviest first, requests in order
-  // of decreasing kv length (each block ranks the requests itself from kv_indptr)
+  // ---- block -> (request, kv head, key split, q block): consecutive block ids go to different
+  // XCDs, the q blocks of one (request, kv head, key split) read the same keys, share an XCD and
+  // run heaviest first, requests in order of decreasing kv length (each block ranks the requests
+  // itself from kv_indptr)
   const int xcd = blockIdx.x & 7;
   const int seq = blockIdx.x >> 3;
-  const int pair = (seq / p.n_qblk) * 8 + xcd;
-  if (pair >= p.n_pairs) return;
+  const int unit = (seq / p.n_qblk) * 8 + xcd;  // (request, kv head, key split)
+  if (unit >= p.n_pairs * p.n_ksplit) return;
+  const int pair = unit / p.n_ksplit;
+  const int split = unit - pair * p.n_ksplit;
   const int qblk = p.n_qblk - 1 - (seq % p.n_qblk);
   const int want_rank = pair / p.n_kv;
   const int kvh = pair - want_rank * p.n_kv;
@@ -109,6 +112,14 @@ __global__ __launch_bounds__(kNW * 64) void prefill_tile256_kernel(PrefillParams
   int k_lo = (p.window > 0) ? max(0, prefix + qi_lo - p.window + 1) : 0;
   k_lo &= ~(kHalf - 1);
   if (k_hi < k_lo) k_hi = k_lo;
+  // key split `split` of n_ksplit: a whole number of step pairs (64 keys) each, the last takes
+  // the ragged end; shares past the end are empty (they still leave a "nothing seen" partial)
+  if (p.n_ksplit > 1) {
+    const int all_pairs = (k_hi - k_lo + 2 * kHalf - 1) / (2 * kHalf);
+    const int share = (all_pairs + p.n_ksplit - 1) / p.n_ksplit * 2 * kHalf;
+    k_lo = min(k_lo + split * share, k_hi);
+    k_hi = min(k_hi, k_lo + share);
+  }
   // steps come in pairs (the loop body handles two, swapping register sets); a half past the
   // end reads clamped keys and is fully masked
   const int n_steps = ((k_hi - k_lo + kHalf - 1) / kHalf + 1) & ~1;
@@ -131,7 +142,8 @@ __global__ __launch_bounds__(kNW * 64) void prefill_tile256_kernel(PrefillParams
     }
     const int qpos = prefix + qi;
     row_lo = (p.window > 0) ? qpos - p.window + 1 : 0;
-    row_hi = p.is_cross ? kn - 1 : min(qpos, kn - 1);
+    // k_hi - 1 only binds under a key split: the pipeline settles one half past its share
+    row_hi = min(p.is_cross ? kn - 1 : min(qpos, kn - 1), k_hi - 1);
     w_lo_max = valid ? row_lo : -0x7fffffff;
     w_hi_min = valid ? row_hi : 0x7fffffff;
     if (!valid) {
@@ -433,6 +445,10 @@ __global__ __launch_bounds__(kNW * 64) void prefill_tile256_kernel(PrefillParams
 #pragma unroll
       for (int kstep = 0; kstep < kKSteps; ++kstep) sa = mfma_32x32x16(k_operand(ks, kstep), qreg[kstep], sa);
     }
+    // Step 0 refills K stage 0 (every later step refills a stage whose readers passed the barrier
+    // at the end of the step before): no wave may start those moves while another still reads
+    // half 0 from it.
+    __syncthreads();
     Stats st_a, st_b;
     settle(sa, needs_mask(k_lo), k_lo, st_a);
 #pragma unroll
@@ -485,8 +501,31 @@ __global__ __launch_bounds__(kNW * 64) void prefill_tile256_kernel(PrefillParams
     __syncthreads();
   }
 
-  // ---- epilogue: normalise, transpose through LDS, store whole rows ---------------------
   // accumulator i of O^T tile dt is dim 32dt + 8(i/4) + 4h + i%4 of query row c32
+  if (p.n_ksplit > 1) {
+    // ---- key split: normalised fp32 partial and log-sum-exp (base 2) per row, from registers
+    float l = l_run;
+    l += __shfl_xor(l, 32, kWave);
+    const float inv = (l > 0.f) ? 1.0f / l : 0.f;
+    const int row = row0 + w * 32 + c32;
+    if (row < rows_total) {
+      const int qi = row / p.group;
+      const int hh = row - qi * p.group;
+      const int64_t at = (int64_t)split * p.part_rows + (int64_t)(q_start + qi) * p.n_q + kvh * p.group + hh;
+      if (h == 0) p.part_lse[at] = (l > 0.f) ? m_run + __log2f(l) : kNegInf;
+      float* dst = p.part_o + at * kD + 4 * h;
+#pragma unroll
+      for (int dt = 0; dt < kDT; ++dt)
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+          f32x4_t v = {oacc[dt][4 * a] * inv, oacc[dt][4 * a + 1] * inv, oacc[dt][4 * a + 2] * inv,
+                       oacc[dt][4 * a + 3] * inv};
+          *reinterpret_cast<f32x4_t*>(dst + 32 * dt + 8 * a) = v;
+        }
+    }
+    return;
+  }
+  // ---- epilogue: normalise, transpose through LDS, store whole rows ---------------------
   unsigned char* os = smem;
   {
     float l = l_run;
@@ -531,7 +570,9 @@ int launch_prefill_tile256(const PrefillArgs& a, hipStream_t stream) {
   const dim3 grid((unsigned)n_blocks);
   if (wide) hipLaunchKernelGGL((prefill_tile256_kernel<true>), grid, dim3(kNW * 64), 0, stream, p);
   else hipLaunchKernelGGL((prefill_tile256_kernel<false>), grid, dim3(kNW * 64), 0, stream, p);
-  return check_launch();
+  const int launched = check_launch();
+  if (launched != MSGL_OK || p.n_ksplit == 1) return launched;
+  return launch_prefill_merge(p, kD, stream);
 }
 
 }  // namespace msgl

@@ -18,6 +18,12 @@ struct PrefillParams {
   int32_t n_qblk, n_pairs;  // q blocks per (request, kv head); batch * n_kv
   int32_t max_len_extend, is_cross, window;
   float scale_log2e;
+  // key splits: each workgroup takes one contiguous share of its rows' visible keys
+  // and leaves a normalised fp32 partial and a base-2 log-sum-exp per row for the merge kernel
+  int32_t n_ksplit;
+  int64_t part_rows;  // total_q * n_q: rows of one split's partial
+  float* part_o;      // [n_ksplit][part_rows][head_dim]
+  float* part_lse;    // [n_ksplit][part_rows]
 #ifdef MSGL_PROFILE_PHASES
   long long* prof;  // [blocks][waves][8] cycle totals
 #endif
@@ -33,6 +39,58 @@ constexpr float kLazy = 8.0f;
 constexpr int kRankedBatch = 128;
 constexpr int kPrefillBlockRows = 256;      // rows per workgroup, head_dim 128
 constexpr int kPrefillBlockRows256 = 128;   // head_dim 256
+// Key splits: when (requests x kv heads x query blocks) cannot fill the chip, the keys of every
+// query block are shared out over several workgroups.
+constexpr int kComputeUnits = 256;
+constexpr int kMaxKeySplits = 32;
+constexpr int kMinKeysPerSplit = 1024;
+
+inline int prefill_block_rows(int64_t head_dim) {
+  return head_dim == 256 ? kPrefillBlockRows256 : kPrefillBlockRows;
+}
+
+// Number of key splits for a launch, from sizes the host knows (the per-request lengths stay on
+// the device: the average visible length stands for all of them).  Cost model: the (request, kv
+// head, split) units are dealt round-robin to the 8 XCDs, a unit brings its query blocks, and an
+// XCD runs its workgroups in rounds of one per compute unit; a split costs a few percent (its
+// partial, the merge).  The count minimises rounds(k) / k * (1 + 0.03 (k - 1)); launches of more
+// than four rounds are left alone.  `forced` > 0 overrides (clamped to kMaxKeySplits).
+inline int prefill_key_splits(int64_t batch, int64_t total_kv, int64_t n_kv, int64_t group,
+                              int64_t max_len_extend, int64_t window, int block_rows,
+                              int64_t forced) {
+  if (forced > 0) return (int)(forced < kMaxKeySplits ? forced : kMaxKeySplits);
+  if (batch <= 0) return 1;
+  constexpr int64_t kXcds = 8, kUnitsPerXcd = kComputeUnits / kXcds;
+  const int64_t n_qblk = (max_len_extend * group + block_rows - 1) / block_rows;
+  const int64_t pairs = batch * n_kv;
+  auto rounds = [&](int64_t k) {
+    const int64_t blocks = (pairs * k + kXcds - 1) / kXcds * n_qblk;  // on the busiest XCD
+    return (blocks + kUnitsPerXcd - 1) / kUnitsPerXcd;
+  };
+  if (n_qblk <= 0 || rounds(1) > 4) return 1;
+  int64_t keys = total_kv / batch;
+  if (window > 0 && keys > window + max_len_extend) keys = window + max_len_extend;
+  int64_t most = keys / kMinKeysPerSplit;
+  if (most > kMaxKeySplits) most = kMaxKeySplits;
+  int best = 1;
+  double best_cost = (double)rounds(1);
+  for (int64_t k = 2; k <= most; ++k) {
+    const double cost = (double)rounds(k) / (double)k * (1.0 + 0.03 * (double)(k - 1));
+    if (cost < best_cost) {
+      best_cost = cost;
+      best = (int)k;
+    }
+  }
+  return best;
+}
+
+inline size_t prefill_split_workspace_bytes(int64_t total_q, int64_t n_q, int64_t head_dim, int n_ksplit) {
+  if (n_ksplit <= 1) return 0;
+  return (size_t)n_ksplit * (size_t)total_q * (size_t)n_q * (size_t)(head_dim + 1) * sizeof(float);
+}
+
+// Combines the partials of a key-split launch into `out` (defined beside the head_dim 128 kernel).
+int launch_prefill_merge(const struct PrefillParams& p, int head_dim, hipStream_t stream);
 
 // Fills `p` and the grid size; returns MSGL_OK, or an error, or sets n_blocks = 0 for an
 // empty problem.  wide: some pool byte offset needs more than 32 bits.
@@ -56,10 +114,15 @@ inline int make_prefill_params(const PrefillArgs& a, PrefillParams& p, int64_t& 
   p.is_cross = a.is_cross;
   p.window = a.window;
   p.scale_log2e = a.sm_scale * 1.4426950408889634f;
+  p.n_ksplit = a.key_splits > 1 ? a.key_splits : 1;
+  p.part_rows = a.total_q * a.n_q;
+  p.part_o = static_cast<float*>(a.workspace);
+  p.part_lse = p.part_o ? p.part_o + (int64_t)p.n_ksplit * p.part_rows * a.head_dim : nullptr;
+  if (p.n_ksplit > 1 && !p.part_o) return MSGL_ERR_WORKSPACE;
   const int64_t rows = (int64_t)a.max_len_extend * p.group;
   const int64_t n_qblk = (rows + block_rows - 1) / block_rows;
   const int64_t n_pairs = a.batch * a.n_kv;
-  n_blocks = (n_pairs + 7) / 8 * 8 * n_qblk;
+  n_blocks = (n_pairs * p.n_ksplit + 7) / 8 * 8 * n_qblk;
   if (n_qblk <= 0 || n_blocks <= 0) {
     n_blocks = 0;
     return MSGL_OK;

@@ -79,6 +79,7 @@ TUNE_SMALLQ_MAXCOLS = 2
 TUNE_PREFILL_VARIANT = 3
 TUNE_SPLITKV_WAVES = 4
 TUNE_GDN_ROWS = 5
+TUNE_PREFILL_KEY_SPLITS = 6
 
 _lib = None
 

@@ -50,10 +50,18 @@ def test_random_prefill_shapes(gpu, seed):
                         kv_lens=kv, extend_lens=ext, pool_factor=rng.choice([1.0, 1.7]),
                         store_new=rng.random() < 0.7, is_cross_attention=is_cross,
                         sliding_window_size=window)
+    # half of the cases force a key split of the tile kernels (the split-K route ignores it)
+    splits = rng.choice([2, 3, 4, 5, 8, 13, 32]) if rng.random() < 0.5 else 0
     what = (f"fuzz prefill seed={seed} heads={n_q}/{n_kv} d={d} page={page} ext={ext} kv={kv} "
-            f"cross={is_cross} W={window}")
+            f"cross={is_cross} W={window} key_splits={splits}")
     print(what, flush=True)
-    got, g = run_gpu(wl, gpu)
+    from mini_sglang_amd_kernel import _lib
+
+    _lib.set_tuning(_lib.TUNE_PREFILL_KEY_SPLITS, splits)
+    try:
+        got, g = run_gpu(wl, gpu)
+    finally:
+        _lib.set_tuning(_lib.TUNE_PREFILL_KEY_SPLITS, 0)
     want, ref = run_oracle(wl)
     assert_close_bf16(got, want, what)
     if wl.out_loc is not None:

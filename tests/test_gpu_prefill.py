@@ -314,3 +314,104 @@ def test_max_len_extend_smaller_than_a_request_leaves_tail_rows_alone(gpu):
                                   g.kv_indices, g.prefix_lens, g.sm_scale, 12)
     torch.cuda.synchronize()
     assert_close_bf16(out.cpu(), want, "reference")
+
+
+# ---- key splits of the tile kernels: a launch with fewer query blocks than compute units shares
+# ---- the keys of every block out over several workgroups and merges fp32 partials ----------------
+@pytest.fixture(params=[2, 3, 7, 32], ids=lambda k: f"{k}splits")
+def key_splits(request):
+    from mini_sglang_amd_kernel import _lib
+
+    _lib.set_tuning(_lib.TUNE_PREFILL_KEY_SPLITS, request.param)
+    yield request.param
+    _lib.set_tuning(_lib.TUNE_PREFILL_KEY_SPLITS, 0)
+
+
+@pytest.mark.parametrize("head_dim", [128, 256])
+@pytest.mark.parametrize("is_cross,window", MASKS)
+def test_key_split_masks(gpu, key_splits, head_dim, is_cross, window):
+    # ragged requests, some with fewer tiles than shares (empty shares), prefix lengths that put
+    # the causal diagonal inside a middle share, windows that start past the first shares
+    wl = build_workload("t", "prefill", seed=700 + head_dim, n_q=8, n_kv=2, head_dim=head_dim,
+                        kv_lens=[70, 300, 64 + 130, 33, 513 + 65, 31, 1000 + 97, 2049 + 300],
+                        extend_lens=[70, 100, 130, 33, 65, 31, 97, 300], pool_factor=1.3,
+                        store_new=True, is_cross_attention=is_cross, sliding_window_size=window)
+    _check(wl, gpu, f"key splits={key_splits} head_dim={head_dim} cross={is_cross} W={window}")
+
+
+@pytest.mark.parametrize("head_dim", [128, 256])
+@pytest.mark.parametrize("n_q,n_kv", [(8, 8), (32, 8), (12, 4), (16, 1)])
+def test_key_split_group_sizes(gpu, key_splits, head_dim, n_q, n_kv):
+    wl = build_workload("t", "prefill", seed=720 + n_q, n_q=n_q, n_kv=n_kv, head_dim=head_dim,
+                        kv_lens=[200 + 96, 129, 1000 + 257, 2100 + 70], extend_lens=[96, 129, 257, 70],
+                        pool_factor=1.2, store_new=True)
+    _check(wl, gpu, f"key splits={key_splits} head_dim={head_dim} n_q={n_q} n_kv={n_kv}")
+
+
+@pytest.mark.parametrize("head_dim", [128, 256])
+def test_key_split_equals_one_pass_and_leaves_capped_rows_alone(gpu, head_dim):
+    """The split result is the one-pass result up to the fp32 merge; rows past max_len_extend
+    keep what `out` held (the merge kernel must not touch them either)."""
+    from mini_sglang_amd_kernel import _lib
+
+    lib = _lib.load()
+    wl = build_workload("t", "prefill", seed=740, n_q=8, n_kv=4, head_dim=head_dim,
+                        kv_lens=[3000 + 90, 5000 + 120, 77], extend_lens=[90, 120, 77],
+                        pool_factor=1.1)
+    g = wl.to(gpu)
+    cap = 100  # request 1 has 120 queries: its last 20 rows stay untouched
+    outs = []
+    for k in (1, 5):
+        print(f"key splits {k} head_dim {head_dim} cap {cap}", flush=True)
+        _lib.set_tuning(_lib.TUNE_PREFILL_KEY_SPLITS, k)
+        try:
+            out = torch.full_like(g.q, 7.0)
+            total_q, n_q, d = g.q.shape
+            batch, total_kv = g.qo_indptr.shape[0] - 1, g.kv_indices.shape[0]
+            ws_bytes = lib.msgl_paged_prefill_workspace_bytes(batch, total_q, total_kv, n_q,
+                                                              g.k_cache.shape[1], d, cap)
+            assert (ws_bytes > 0) == (k > 1)
+            ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=gpu)
+            rc = lib.msgl_paged_prefill_attention(
+                g.q.data_ptr(), g.k_cache.data_ptr(), g.v_cache.data_ptr(), g.qo_indptr.data_ptr(),
+                g.kv_indptr.data_ptr(), g.kv_indices.data_ptr(), g.prefix_lens.data_ptr(),
+                out.data_ptr(), ws.data_ptr(), ws_bytes, batch, total_q, total_kv, n_q,
+                g.k_cache.shape[1], d, g.k_cache.shape[0], g.k_cache.stride(0), g.v_cache.stride(0),
+                float(g.sm_scale), cap, 0, 0, 0, None)
+            assert rc == 0, _lib.strerror(rc)
+            if k > 1:  # too small a workspace is refused, not overrun
+                assert lib.msgl_paged_prefill_attention(
+                    g.q.data_ptr(), g.k_cache.data_ptr(), g.v_cache.data_ptr(), g.qo_indptr.data_ptr(),
+                    g.kv_indptr.data_ptr(), g.kv_indices.data_ptr(), g.prefix_lens.data_ptr(),
+                    out.data_ptr(), ws.data_ptr(), ws_bytes - 1, batch, total_q, total_kv, n_q,
+                    g.k_cache.shape[1], d, g.k_cache.shape[0], g.k_cache.stride(0),
+                    g.v_cache.stride(0), float(g.sm_scale), cap, 0, 0, 0, None) == -8
+            torch.cuda.synchronize()
+        finally:
+            _lib.set_tuning(_lib.TUNE_PREFILL_KEY_SPLITS, 0)
+        outs.append(out.cpu())
+    tail = slice(90 + cap, 90 + 120)
+    for out in outs:
+        assert (out[tail].float() == 7.0).all()
+    assert_close_bf16(outs[1], outs[0].float(), "split vs one pass", max_tol=8e-3, mean_tol=4e-4)
+    want, _ = run_oracle(wl)
+    keep = torch.ones(want.shape[0], dtype=torch.bool)
+    keep[tail] = False
+    assert_close_bf16(outs[1][keep], want[keep], "split vs oracle")
+
+
+@pytest.mark.parametrize("head_dim", [128, 256])
+@pytest.mark.parametrize("extend", [70, 300])
+def test_one_long_request_splits_its_keys_by_itself(gpu, head_dim, extend):
+    """No knob: one request with a long prefix has too few query blocks for the chip, so the
+    library asks for a workspace and splits."""
+    from mini_sglang_amd_kernel import _lib
+
+    lib = _lib.load()
+    n_q, n_kv, prefix = 8, 2, 20000
+    assert lib.msgl_paged_prefill_workspace_bytes(1, extend, prefix + extend, n_q, n_kv, head_dim, extend) > 0
+    # the benchmark's extend shape fills the chip and needs none
+    assert lib.msgl_paged_prefill_workspace_bytes(8, 8 * 512, 8 * 8704, 32, 8, head_dim, 512) == 0
+    wl = build_workload("t", "prefill", seed=760 + extend, n_q=n_q, n_kv=n_kv, head_dim=head_dim,
+                        kv_lens=[prefix + extend], extend_lens=[extend], pool_factor=1.1, store_new=True)
+    _check(wl, gpu, f"one long request head_dim={head_dim} extend={extend}")
