@@ -1,0 +1,81 @@
+"""Same inputs, same bits: every attention route is launched many times on one workload and each
+result must equal the first bit for bit.  The kernels use no atomics and merge partials in a fixed
+order, so any difference is a race between waves (a stage refilled while another wave still reads
+it, a wait that does not cover a load), which the parity tests only see when it happens to strike
+on their single run."""
+import pytest
+import torch
+
+from mini_sglang_amd.workloads import build_workload
+from mini_sglang_amd_kernel import _lib, paged_decode_attention, paged_prefill_attention
+
+pytestmark = pytest.mark.gpu
+
+RUNS = 40
+
+
+def _prefill(g, cap, **kw):
+    return paged_prefill_attention(g.q, g.k_cache, g.v_cache, g.qo_indptr, g.kv_indptr, g.kv_indices,
+                                   g.prefix_lens, g.sm_scale, cap, **kw)
+
+
+@pytest.mark.parametrize("head_dim", [128, 256])
+@pytest.mark.parametrize("splits", [1, 4, 32])
+@pytest.mark.parametrize("n_q,n_kv", [(32, 8), (16, 1)])
+def test_tile_kernels_repeat_bit_identical(gpu, head_dim, splits, n_q, n_kv):
+    # many workgroups with few pipeline steps each: start-up and wind-down of the stage rings
+    # are most of what runs
+    wl = build_workload("t", "prefill", seed=900 + n_q, n_q=n_q, n_kv=n_kv, head_dim=head_dim,
+                        kv_lens=[200 + 96, 129, 1000 + 257, 2100 + 70, 33, 64 + 65],
+                        extend_lens=[96, 129, 257, 70, 33, 65], pool_factor=1.2)
+    g = wl.to(gpu)
+    print(f"repeat tile head_dim={head_dim} splits={splits} heads={n_q}/{n_kv}", flush=True)
+    _lib.set_tuning(_lib.TUNE_PREFILL_KEY_SPLITS, splits)
+    try:
+        outs = [_prefill(g, 257) for _ in range(RUNS)]
+        torch.cuda.synchronize()
+    finally:
+        _lib.set_tuning(_lib.TUNE_PREFILL_KEY_SPLITS, 0)
+    for i, out in enumerate(outs[1:], 1):
+        assert torch.equal(out.view(torch.int16), outs[0].view(torch.int16)), f"run {i} differs from run 0"
+
+
+@pytest.mark.parametrize("head_dim", [128, 256])
+@pytest.mark.parametrize("is_cross,window", [(False, 0), (False, 100), (True, 0)])
+def test_tile_kernels_repeat_bit_identical_long_rows(gpu, head_dim, is_cross, window):
+    wl = build_workload("t", "prefill", seed=910, n_q=8, n_kv=2, head_dim=head_dim,
+                        kv_lens=[3000 + 300, 31, 700 + 513], extend_lens=[300, 31, 513],
+                        pool_factor=1.1, is_cross_attention=is_cross, sliding_window_size=window)
+    g = wl.to(gpu)
+    print(f"repeat tile long head_dim={head_dim} cross={is_cross} W={window}", flush=True)
+    outs = [_prefill(g, 513, is_cross_attention=is_cross, sliding_window_size=window) for _ in range(RUNS)]
+    torch.cuda.synchronize()
+    for i, out in enumerate(outs[1:], 1):
+        assert torch.equal(out.view(torch.int16), outs[0].view(torch.int16)), f"run {i} differs from run 0"
+
+
+@pytest.mark.parametrize("head_dim", [128, 256])
+@pytest.mark.parametrize("q_len", [1, 4, 8])
+def test_splitk_kernel_repeat_bit_identical(gpu, head_dim, q_len):
+    lens = [1, 17, 900, 4000, 64, 2500, 129, 33]
+    wl = build_workload("t", "prefill", seed=920, n_q=16, n_kv=4, head_dim=head_dim,
+                        kv_lens=[n + q_len for n in lens], extend_lens=[q_len] * len(lens), pool_factor=1.1)
+    g = wl.to(gpu)
+    print(f"repeat split-K head_dim={head_dim} q_len={q_len}", flush=True)
+    outs = [_prefill(g, q_len) for _ in range(RUNS)]
+    torch.cuda.synchronize()
+    for i, out in enumerate(outs[1:], 1):
+        assert torch.equal(out.view(torch.int16), outs[0].view(torch.int16)), f"run {i} differs from run 0"
+
+
+@pytest.mark.parametrize("head_dim", [128, 256])
+def test_decode_repeat_bit_identical(gpu, head_dim):
+    wl = build_workload("t", "decode", seed=930, n_q=32, n_kv=8, head_dim=head_dim,
+                        kv_lens=[1, 17, 900, 4000, 64, 2500, 129, 33, 7000, 2, 640], pool_factor=1.1)
+    g = wl.to(gpu)
+    print(f"repeat decode head_dim={head_dim}", flush=True)
+    outs = [paged_decode_attention(g.q, g.k_cache, g.v_cache, g.kv_indptr, g.kv_indices,
+                                   g.num_kv_splits, g.sm_scale, g.max_kv_splits) for _ in range(RUNS)]
+    torch.cuda.synchronize()
+    for i, out in enumerate(outs[1:], 1):
+        assert torch.equal(out.view(torch.int16), outs[0].view(torch.int16)), f"run {i} differs from run 0"
