@@ -79,3 +79,25 @@ def test_decode_repeat_bit_identical(gpu, head_dim):
     torch.cuda.synchronize()
     for i, out in enumerate(outs[1:], 1):
         assert torch.equal(out.view(torch.int16), outs[0].view(torch.int16)), f"run {i} differs from run 0"
+
+
+@pytest.mark.parametrize("cfg,variant,head_dim", [(2, "", 128), (3, "", 128), (3, "", 256), (5, "", 128),
+                                                  (5, "window", 128)])
+def test_benchmark_shapes_repeat_bit_identical(gpu, cfg, variant, head_dim):
+    """The same demand at full size, where every compute unit is busy and waves drift apart."""
+    from _gpu_util import run_gpu
+    from mini_sglang_amd.workloads import config_workload
+
+    wl = config_workload(cfg, variant=variant, pool_device=gpu, head_dim=head_dim)
+    print(f"repeat shape {cfg} {variant} head_dim={head_dim}", flush=True)
+    first, g = run_gpu(wl, gpu)
+    first = first.view(torch.int16)
+    for i in range(1, 16):
+        if wl.kind == "decode":
+            out = paged_decode_attention(g.q, g.k_cache, g.v_cache, g.kv_indptr, g.kv_indices,
+                                         g.num_kv_splits, g.sm_scale, g.max_kv_splits)
+        else:
+            out = _prefill(g, g.max_len_extend, is_cross_attention=g.is_cross_attention,
+                           sliding_window_size=g.sliding_window_size)
+        torch.cuda.synchronize()
+        assert torch.equal(out.cpu().view(torch.int16), first), f"run {i} differs from run 0"
