@@ -427,6 +427,51 @@ def run_radix_cache(cpu_baseline: bool):
     return row
 
 
+def run_small_launch_extends(dev, steps: int, warmup: int):
+    """Extends too small to fill the chip (one long request, a short chunk): the tile kernels with
+    their keys in one pass (knob 1) against the library's own choice of key splits.  Not a BASELINE
+    shape; shows what the split buys and that both give the same result."""
+    import torch
+
+    from mini_sglang_amd.workloads import build_workload
+    from mini_sglang_amd_kernel import _lib, paged_prefill_attention
+
+    rows = []
+    for name, prefix, extend, n_q, n_kv, d in (
+            ("one_request_128k_context_1024_extend", 130048, 1024, 16, 4, 128),
+            ("one_request_128k_context_1024_extend_head_dim_256", 130048, 1024, 16, 4, 256),
+            ("one_request_32k_context_512_extend", 32768, 512, 32, 8, 128),
+            ("one_request_8k_context_64_extend", 8192, 64, 32, 8, 128)):
+        wl = build_workload(name, "prefill", seed=7, n_q=n_q, n_kv=n_kv, head_dim=d,
+                            kv_lens=[prefix + extend], extend_lens=[extend], pool_factor=1.0,
+                            pool_device=dev)
+        g = wl.to(dev)
+
+        def step():
+            return paged_prefill_attention(g.q, g.k_cache, g.v_cache, g.qo_indptr, g.kv_indptr,
+                                           g.kv_indices, g.prefix_lens, g.sm_scale, extend)
+        row = {"sizes": name, "n_q": n_q, "n_kv": n_kv, "head_dim": d,
+               "algorithmic_flops": wl.attention_flops()}
+        outs = {}
+        for label, knob in (("one_pass", 1), ("key_split", 0)):
+            _lib.set_tuning(_lib.TUNE_PREFILL_KEY_SPLITS, knob)
+            try:
+                ms, _, _ = time_steps(step, max(3, steps // 5), max(1, warmup // 5))
+                outs[label] = step().float()
+                torch.cuda.synchronize()
+            finally:
+                _lib.set_tuning(_lib.TUNE_PREFILL_KEY_SPLITS, 0)
+            row[label + "_us"] = ms * 1e3
+            row[label + "_TFLOPs"] = row["algorithmic_flops"] / (ms * 1e-3) / 1e12
+        row["max_abs_diff"] = float((outs["one_pass"] - outs["key_split"]).abs().max())
+        log(f"[small launch] {name}: one pass {row['one_pass_us']:.0f} us, key split "
+            f"{row['key_split_us']:.0f} us ({row['key_split_TFLOPs']:.0f} TFLOP/s), "
+            f"max diff {row['max_abs_diff']:.1e}")
+        rows.append(row)
+        del g, wl
+    return rows
+
+
 def mfma_rate_probe():
     """Sustained v_mfma_f32_32x32x16_bf16 rate of the whole chip on register-resident operands,
     nothing else running: all-zero operands and N(0,1) operands that change every instruction.
@@ -580,6 +625,7 @@ def main():
         result["metadata_build"] = run_metadata_build(dev, args.steps, args.warmup,
                                                       not args.no_cpu_baseline)
         result["radix_prefix_cache"] = run_radix_cache(not args.no_cpu_baseline)
+        result["small_launch_extends"] = run_small_launch_extends(dev, args.steps, args.warmup)
     result["all_configs"] = rows
     print(json.dumps(result))
 
