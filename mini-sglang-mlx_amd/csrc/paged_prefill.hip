@@ -36,14 +36,6 @@
 namespace msgl {
 namespace {
 
-#ifdef MSGL_PROFILE_PHASES
-#define MSGL_TICK(i) do { const long long t_ = clock64(); prof_acc[i] += t_ - prof_t; prof_t = t_; } while (0)
-#define MSGL_PROF_HALF(x) prof_half = (x)
-#else
-#define MSGL_TICK(i) do { } while (0)
-#define MSGL_PROF_HALF(x) do { } while (0)
-#endif
-
 constexpr int kUnitRows = 4;                 // rows moved by one LDS-direct load
 constexpr int kUnits = kBN / kUnitRows;      // 16 per tile
 constexpr int kKUnit = 1024 + 16;            // bytes between K units
@@ -235,11 +227,6 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
   const uint32_t v_lane = (uint32_t)(4 * h + ((lane & 15) >> 2)) * kVUnit +
                           (uint32_t)((lane >> 4) & 1) * 32u + (uint32_t)(lane & 3) * 8u;
 
-#ifdef MSGL_PROFILE_PHASES
-  long long prof_acc[16] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-  long long prof_t = 0;
-  int prof_half = 0;
-#endif
   // ---- the pieces of one half tile (32 keys) ----------------------------------------------
   struct Scores {
     f32x16_t s[RT];  // S^T[key][row]: key = base + 8(i/4) + 4h + i%4, row = 32rt + c32
@@ -403,7 +390,6 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
     qk_slice(0, kops);
     exp_slice(0);
     side(0);
-    MSGL_TICK(8 + 4 * prof_half + 0);
     __builtin_amdgcn_sched_barrier(0);
     // slice 1
 #pragma unroll
@@ -412,7 +398,6 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
     exp_slice(8);
     pack_slice(0);
     side(1);
-    MSGL_TICK(8 + 4 * prof_half + 1);
     __builtin_amdgcn_sched_barrier(0);
     st_nxt.mul = p.scale_log2e;
     if (mask_nxt) {  // boundary half: scale and mask in place
@@ -432,7 +417,6 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) pin(mx[rt]);
     side(2);
-    MSGL_TICK(8 + 4 * prof_half + 2);
     __builtin_amdgcn_sched_barrier(0);
     // slice 3
 #pragma unroll
@@ -442,7 +426,6 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
     for (int rt = 0; rt < RT; ++rt) l_run[rt] = l_run[rt] * st_cur.alpha[rt] + psum[rt];
     decide(mx, st_nxt);
     side(3);
-    MSGL_TICK(8 + 4 * prof_half + 3);
     __builtin_amdgcn_sched_barrier(0);
   };
 
@@ -499,10 +482,6 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
     bf16x8_t kops[4];
 #pragma unroll
     for (int e = 0; e < 4; ++e) kops[e] = k_operand(smem + k_cur + k_lane + 512, e);
-#ifdef MSGL_PROFILE_PHASES
-    prof_t = clock64();
-    const long long prof_c0 = prof_t, prof_w0 = wall_clock64();
-#endif
     for (int j = 0; j < n_tiles; ++j) {
       const int tb = k_lo + j * kBN;
       // the moves of this iteration (V of tile j+1, K of tile j+2) are issued one per slice
@@ -510,9 +489,7 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
       // used in the next iteration
       offsets_from_slots();
       slot_load(tb + 3 * kBN);
-      MSGL_TICK(0);
       // half (j,0): scores of (j,1) from K of tile j, P V of (j-1,1) from V of tile j-1
-      MSGL_PROF_HALF(0);
       rescale(st_b.alpha);
       fused_half(sa, st_a, sb, st_b, needs_mask(tb + 32), tb + 32, smem + k_cur + k_lane + 512,
                  smem + v_prev + v_lane + 512, smem + k_next + k_lane, kops, pb_b, pb_a,
@@ -522,17 +499,12 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
                    for (int n = sl * PER; n < (sl + 1) * PER; ++n) move(n, k_fill, v_fill);
                  });
       rotate_v_offsets();
-      MSGL_TICK(1);
-      MSGL_PROF_HALF(1);
       // half (j,1): scores of (j+1,0) from K of tile j+1, P V of (j,0) from V of tile j
       rescale(st_a.alpha);
       fused_half(sb, st_b, sa, st_a, needs_mask(tb + 64), tb + 64, smem + k_next + k_lane,
                  smem + v_cur + v_lane, smem + k_next + k_lane + 512, kops, pb_a, pb_b, [](int) {});
-      MSGL_TICK(2);
       wait_all_vm();
-      MSGL_TICK(3);
       __syncthreads();
-      MSGL_TICK(4);
       const uint32_t k_freed = k_cur;
       k_cur = k_next;
       k_next = k_fill;
@@ -546,16 +518,6 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
     rescale(st_b.alpha);
     pv_half(v_prev, 1, pb_b);
     __syncthreads();  // the epilogue reuses the stages as its output staging area
-#ifdef MSGL_PROFILE_PHASES
-    if (lane == 0) {
-      long long* dst = p.prof + ((long long)blockIdx.x * 8 + w) * 16;
-      for (int i = 0; i < 5; ++i) dst[i] = prof_acc[i];
-      dst[5] = n_tiles;
-      dst[6] = clock64() - prof_c0;
-      dst[7] = wall_clock64() - prof_w0;
-      for (int i = 8; i < 16; ++i) dst[i] = prof_acc[i];
-    }
-#endif
   }
 
   // accumulator i of O^T tile dt is dim 32dt + 8(i/4) + 4h + i%4 of query row c32
@@ -679,10 +641,6 @@ int launch_prefill_merge(const PrefillParams& p, int head_dim, hipStream_t strea
   return check_launch();
 }
 
-#ifdef MSGL_PROFILE_PHASES
-static long long* g_prof_buf = nullptr;
-extern "C" __attribute__((visibility("default"))) long long* msgl_debug_prof_buffer() { return g_prof_buf; }
-#endif
 static std::atomic<int> g_tile_variant{0};
 int tile_variant() { return g_tile_variant.load(); }
 void set_tile_variant(int v) { g_tile_variant.store(v); }
@@ -694,12 +652,6 @@ int launch_prefill_tile(const PrefillArgs& a, hipStream_t stream) {
   bool wide = false;
   const int rc = make_prefill_params(a, p, n_blocks, wide);
   if (rc != MSGL_OK || n_blocks == 0) return rc;
-#ifdef MSGL_PROFILE_PHASES
-  static long long* prof_buf = nullptr;
-  if (!prof_buf) (void)hipMalloc(&prof_buf, 8192 * 128 * sizeof(long long));
-  p.prof = prof_buf;
-  g_prof_buf = prof_buf;
-#endif
   const dim3 grid((unsigned)n_blocks);
   if (tile_variant() == 1) {
     if (wide) hipLaunchKernelGGL((prefill_tile_kernel<128, 2, 4, true>), grid, dim3(256), 0, stream, p);

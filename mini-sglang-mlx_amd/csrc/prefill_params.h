@@ -24,9 +24,6 @@ struct PrefillParams {
   int64_t part_rows;  // total_q * n_q: rows of one split's partial
   float* part_o;      // [n_ksplit][part_rows][head_dim]
   float* part_lse;    // [n_ksplit][part_rows]
-#ifdef MSGL_PROFILE_PHASES
-  long long* prof;  // [blocks][waves][8] cycle totals
-#endif
 };
 
 constexpr int kBN = 64;  // keys per tile
