@@ -122,7 +122,9 @@ MSGL_API int msgl_paged_decode_attention(const void* q, const void* k_cache, con
 /*
  * Workspace (bytes) that msgl_paged_prefill_attention needs for these sizes: the partials of the
  * split-K route, or those of the tile kernels when the launch is too small to fill the chip and
- * the keys of each query block are shared out over several workgroups; 0 otherwise.
+ * the keys of each query block are shared out over several workgroups; 0 otherwise.  The split-K
+ * route needs its workspace (MSGL_ERR_WORKSPACE without it); the tile kernels fall back to one
+ * pass over the keys when the workspace is missing or too small.
  */
 MSGL_API size_t msgl_paged_prefill_workspace_bytes(int64_t batch, int64_t total_q, int64_t total_kv,
                                           int64_t num_q_heads, int64_t num_kv_heads,

@@ -302,9 +302,10 @@ int msgl_paged_prefill_attention(const void* q, const void* k_cache, const void*
                                           sliding_window_size, msgl::prefill_block_rows(head_dim),
                                           g_key_splits.load());
   if (a.key_splits > 1) {
+    // the split is an optimisation: without room for its partials the keys go in one pass
     const size_t need = msgl::prefill_split_workspace_bytes(total_q, num_q_heads, head_dim, a.key_splits);
-    if (!workspace || workspace_bytes < need || !aligned16(workspace)) return MSGL_ERR_WORKSPACE;
-    a.workspace = workspace;
+    if (!workspace || workspace_bytes < need || !aligned16(workspace)) a.key_splits = 1;
+    else a.workspace = workspace;
   }
   return head_dim == 256 ? msgl::launch_prefill_tile256(a, s) : msgl::launch_prefill_tile(a, s);
 }
