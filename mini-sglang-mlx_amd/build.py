@@ -3,7 +3,8 @@
 Usage: ``python build.py [--force]``.  hipcc cross-compiles, so this runs without a GPU.
 Each ``.hip`` file is compiled to an object on its own (in parallel) and the objects are
 linked into one shared library whose only exported symbols are the ``msgl_*`` C ABI of
-``include/msgl_paged_attention.h`` and ``include/msgl_radix_cache.h``.
+``include/msgl_paged_attention.h``, ``include/msgl_radix_cache.h`` and
+``include/msgl_state_pool.h``.
 """
 from __future__ import annotations
 
@@ -22,7 +23,7 @@ PROBE_SRC = os.path.join(CSRC, "probes", "mfma_rate_probe.hip")
 PROBE_PATH = os.path.join(LIB_DIR, "libmsgl_probes.so")
 SOURCES = ["api.hip", "store_kv_cache.hip", "paged_splitkv.hip", "paged_prefill.hip", "paged_prefill_d256.hip",
            "build_metadata.hip", "qk_norm_rope_store.hip",
-           "gdn_state.hip", "radix_cache.hip"]
+           "gdn_state.hip", "radix_cache.hip", "state_slots.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # Packed fp32 VALU forms are switched off for every device compile on this target.
@@ -61,6 +62,7 @@ def build(force: bool = False, save_temps: bool = False) -> str:
     headers = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".h")]
     headers.append(os.path.join(HERE, "..", "include", "msgl_paged_attention.h"))
     headers.append(os.path.join(HERE, "..", "include", "msgl_radix_cache.h"))
+    headers.append(os.path.join(HERE, "..", "include", "msgl_state_pool.h"))
     todo = []
     for src in SOURCES:
         obj = os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o")

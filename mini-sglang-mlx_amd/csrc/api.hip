@@ -310,6 +310,18 @@ int msgl_paged_prefill_attention(const void* q, const void* k_cache, const void*
   return head_dim == 256 ? msgl::launch_prefill_tile256(a, s) : msgl::launch_prefill_tile(a, s);
 }
 
+int msgl_copy_state_slots(void* slab, int64_t layer_stride_bytes, int64_t slot_stride_bytes,
+                          int64_t row_bytes, int64_t n_layers, int64_t num_slots, const int32_t* src,
+                          const int32_t* dst, int64_t n_pairs, void* stream) {
+  if (n_layers < 0 || num_slots < 0 || n_pairs < 0 || row_bytes < 0 || slot_stride_bytes < row_bytes ||
+      (n_layers > 1 && layer_stride_bytes < num_slots * slot_stride_bytes))
+    return MSGL_ERR_SHAPE;
+  if (n_layers == 0 || n_pairs == 0 || row_bytes == 0) return MSGL_OK;
+  if (!slab || !dst) return MSGL_ERR_NULL_POINTER;
+  return msgl::launch_state_slots(slab, layer_stride_bytes, slot_stride_bytes, row_bytes, n_layers,
+                                  num_slots, src, dst, n_pairs, static_cast<hipStream_t>(stream));
+}
+
 int msgl_build_attention_metadata(const int32_t* page_table, int64_t table_stride0,
                                   int64_t n_table_rows, int64_t max_seq_len,
                                   const int32_t* table_rows, const int32_t* kv_lens,

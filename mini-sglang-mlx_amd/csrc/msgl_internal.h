@@ -6,6 +6,7 @@
 #include <stdint.h>
 
 #include "../../include/msgl_paged_attention.h"
+#include "../../include/msgl_state_pool.h"
 
 namespace msgl {
 
@@ -135,6 +136,12 @@ struct GdnArgs {
 int launch_gdn_state(const GdnArgs& a, hipStream_t stream);
 // benchmarking switch: state rows per 16-lane group (1, 2, 4; 0 = chosen from the problem size)
 void gdn_set_rows(int v);
+
+// ---- state_slots.hip -------------------------------------------------------------------
+// src == nullptr: zero fill of the dst slots
+int launch_state_slots(void* base, int64_t layer_stride, int64_t slot_stride, int64_t row_bytes,
+                       int64_t n_layers, int64_t num_slots, const int32_t* src, const int32_t* dst,
+                       int64_t n_pairs, hipStream_t stream);
 
 inline int check_launch() { return hipGetLastError() == hipSuccess ? MSGL_OK : MSGL_ERR_LAUNCH; }
 

@@ -1,5 +1,5 @@
-"""ctypes binding of ``libmsgl_paged_attention.so`` (the C ABI in ``include/msgl_paged_attention.h``
-and ``include/msgl_radix_cache.h``).
+"""ctypes binding of ``libmsgl_paged_attention.so`` (the C ABI in ``include/msgl_paged_attention.h``,
+``include/msgl_radix_cache.h`` and ``include/msgl_state_pool.h``).
 
 The library is built in-tree by ``mini-sglang-mlx_amd/build.py``; nothing here compiles at
 import time and nothing falls back to another implementation: a missing library is an
@@ -49,6 +49,8 @@ SIGNATURES = {
         ctypes.c_int,
         [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64,
          _i64, _i64, _i64, _i64, _i32, _vp]),
+    # include/msgl_state_pool.h (recurrent-state pool)
+    "msgl_copy_state_slots": (ctypes.c_int, [_vp, _i64, _i64, _i64, _i64, _i64, _vp, _vp, _i64, _vp]),
     # include/msgl_radix_cache.h (host-side prefix cache)
     "msgl_fast_compare_key": (_sz, [_vp, _sz, _vp, _sz, _i32, _vp]),
     "msgl_radix_create": (_vp, []),
