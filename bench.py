@@ -371,6 +371,62 @@ def run_gdn_state(dev, steps: int, warmup: int, cpu_baseline: bool):
     return rows_out
 
 
+def run_state_pool(dev, steps: int, warmup: int, cpu_baseline: bool):
+    """Recurrent-state pool: the batched slot copy that seeds every request's scratch slot from its
+    main slot before a replay-style verify, at the gdn benchmark's state size (hv 32, dk = dv = 128
+    fp32 = 2 MiB per slot and layer, plus a (3, 8192) bf16 conv state) for 24 layers.  HBM-bound:
+    every copied byte is read once and written once."""
+    import torch
+
+    from mini_sglang_amd.kvcache import MambaStateConfig, MambaStatePool
+
+    layers, hv, d = 24, 32, 128
+    rows_out = []
+    for name, batch in (("verify_seed_8_requests", 8), ("verify_seed_32_requests", 32)):
+        pool = MambaStatePool(MambaStateConfig(num_slots=2 * batch, num_layers=layers,
+                                               conv_shapes=[[(3, 8192)]] * layers,
+                                               temporal_shapes=[(hv, d, d)] * layers), device=dev)
+        for l in range(layers):
+            pool.temporal_state(l).normal_()
+        src = torch.arange(1, batch + 1, dtype=torch.int32, device=dev)
+        dst = torch.arange(batch + 1, 2 * batch + 1, dtype=torch.int32, device=dev)
+
+        def step():
+            pool.copy_batched(src, dst)
+
+        step()
+        torch.cuda.synchronize()
+        mean_ms, per, _ = time_steps(step, steps, warmup)
+        per_slot = layers * (hv * d * d * 4 + 3 * 8192 * 2)
+        moved = 2 * batch * per_slot
+        exact = all(torch.equal(pool.temporal_state(l)[1:batch + 1], pool.temporal_state(l)[batch + 1:])
+                    for l in (0, layers - 1))
+        row = {"sizes": name, "pairs": batch, "layers": layers, "us_mean": mean_ms * 1e3,
+               "us_min": min(per) * 1e3, "algorithmic_bytes": moved,
+               "achieved_GBps": moved / (mean_ms * 1e-3) / 1e9,
+               "hbm_frac": moved / (mean_ms * 1e-3) / 8e12, "bit_exact": exact}
+        if cpu_baseline:
+            import numpy as np
+
+            from oracle.mamba_pool_oracle import MambaPoolOracle  # checker and CPU baseline only
+
+            n_layers = 2  # bounded sample
+            ref = MambaPoolOracle(2 * batch, n_layers, [[(3, 8192)]] * n_layers, [(hv, d, d)] * n_layers)
+            for t in ref.temporal:
+                t[...] = 1.0
+            t1 = time.perf_counter()
+            ref.copy_batched(np.arange(1, batch + 1), np.arange(batch + 1, 2 * batch + 1))
+            dt = time.perf_counter() - t1
+            row["cpu_port_GBps"] = moved * n_layers / layers / dt / 1e9
+            row["cpu_sample"] = f"{n_layers} of {layers} layers, numpy port, 1 core"
+        log(f"[state pool] {name}: {row['us_mean']:.1f} us mean ({row['us_min']:.1f} min)  "
+            f"{row['achieved_GBps']:.0f} GB/s ({row['hbm_frac']*100:.1f}% of hbm peak)  "
+            f"cpu {row.get('cpu_port_GBps', float('nan')):.2f} GB/s  bit exact {exact}")
+        rows_out.append(row)
+        del pool
+    return rows_out
+
+
 def run_radix_cache(cpu_baseline: bool):
     """Host-side prefix cache: 2048 finished requests (one of 8 shared 1024-token system prompts
     plus a 512-token body of their own) are inserted, then every request comes back with 64 new
@@ -625,6 +681,7 @@ def main():
         result["metadata_build"] = run_metadata_build(dev, args.steps, args.warmup,
                                                       not args.no_cpu_baseline)
         result["radix_prefix_cache"] = run_radix_cache(not args.no_cpu_baseline)
+        result["state_pool_copy"] = run_state_pool(dev, args.steps, args.warmup, not args.no_cpu_baseline)
         result["small_launch_extends"] = run_small_launch_extends(dev, args.steps, args.warmup)
     result["all_configs"] = rows
     print(json.dumps(result))
