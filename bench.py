@@ -427,6 +427,59 @@ def run_state_pool(dev, steps: int, warmup: int, cpu_baseline: bool):
     return rows_out
 
 
+def run_decode_step_graph(dev, steps: int, warmup: int):
+    """One decode step of one layer at shape 1's sizes (metadata build -> fused norm + rope + store
+    -> decode attention: launch-bound), issued eagerly from Python and replayed from a HIP graph
+    captured once.  Both run the same kernels on the same buffers."""
+    import torch
+
+    from mini_sglang_amd_kernel import (build_attention_metadata, paged_decode_attention,
+                                        qk_norm_rope_store)
+
+    n_q, n_kv, d, max_seq, slots = 16, 8, 128, 2048, 16384
+    lens = [37, 128, 500, 1023]
+    b = len(lens)
+    g = torch.Generator().manual_seed(0x5EED0400)
+    bf = lambda *s: torch.randn(s, generator=g).to(dev, torch.bfloat16)
+    kc, vc, q, k, v = bf(slots, n_kv, d), bf(slots, n_kv, d), bf(b, n_q, d), bf(b, n_kv, d), bf(b, n_kv, d)
+    qw, kw = torch.ones(d, dtype=torch.bfloat16, device=dev), torch.ones(d, dtype=torch.bfloat16, device=dev)
+    table = torch.randperm(slots, generator=g)[:b * max_seq].to(torch.int32).view(b, max_seq).to(dev)
+    rows = torch.arange(b, dtype=torch.int32, device=dev)
+    start = torch.tensor(lens, dtype=torch.int32, device=dev)
+    kv_lens = start.clone()
+    out = torch.zeros(b, n_q, d, dtype=torch.bfloat16, device=dev)
+
+    def step():
+        meta = build_attention_metadata(table, rows, kv_lens, total_kv=b * max_seq)
+        out_loc = table[rows.long(), (kv_lens - 1).long()]
+        q_rot = qk_norm_rope_store(q, k, v, qw, kw, meta["positions"], out_loc, kc, vc, eps=1e-6,
+                                   rope_base=1e6)
+        out.copy_(paged_decode_attention(q_rot, kc, vc, meta["kv_indptr"], meta["kv_indices"],
+                                         meta["num_kv_splits"], d ** -0.5, 32))
+
+    side = torch.cuda.Stream(device=dev)
+    side.wait_stream(torch.cuda.current_stream(dev))
+    with torch.cuda.stream(side):
+        step()
+    torch.cuda.current_stream(dev).wait_stream(side)
+    torch.cuda.synchronize()
+    eager_ms, _, eager_wall = time_steps(step, steps, warmup)
+    want = out.clone()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    out.zero_()
+    graph_ms, _, graph_wall = time_steps(graph.replay, steps, warmup)
+    torch.cuda.synchronize()
+    row = {"sizes": "shape1_decode_step_one_layer", "batch": b, "eager_us": eager_ms * 1e3,
+           "eager_wall_us": eager_wall / steps * 1e3, "graph_replay_us": graph_ms * 1e3,
+           "graph_replay_wall_us": graph_wall / steps * 1e3, "same_bits": bool(torch.equal(out, want))}
+    log(f"[decode step] eager {row['eager_us']:.1f} us on the device ({row['eager_wall_us']:.1f} wall), "
+        f"graph replay {row['graph_replay_us']:.1f} us ({row['graph_replay_wall_us']:.1f} wall), "
+        f"same bits {row['same_bits']}")
+    return row
+
+
 def run_radix_cache(cpu_baseline: bool):
     """Host-side prefix cache: 2048 finished requests (one of 8 shared 1024-token system prompts
     plus a 512-token body of their own) are inserted, then every request comes back with 64 new
@@ -681,6 +734,7 @@ def main():
         result["metadata_build"] = run_metadata_build(dev, args.steps, args.warmup,
                                                       not args.no_cpu_baseline)
         result["radix_prefix_cache"] = run_radix_cache(not args.no_cpu_baseline)
+        result["decode_step_graph"] = run_decode_step_graph(dev, args.steps, args.warmup)
         result["state_pool_copy"] = run_state_pool(dev, args.steps, args.warmup, not args.no_cpu_baseline)
         result["small_launch_extends"] = run_small_launch_extends(dev, args.steps, args.warmup)
     result["all_configs"] = rows
