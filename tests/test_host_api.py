@@ -76,6 +76,24 @@ def test_c_abi_argument_checks_return_codes_without_touching_a_gpu():
     assert lib.msgl_set_tuning(99, 1) == -9
     assert lib.msgl_paged_decode_workspace_bytes(4, 1000, 32, 8, 128) > 0
     assert lib.msgl_paged_decode_workspace_bytes(4, 1000, 30, 8, 128) == 0
+    # prefill workspace: none for a launch that fills the chip, the partials of a key split for
+    # one long request, none again when splitting is switched off
+    assert lib.msgl_paged_prefill_workspace_bytes(8, 4096, 8 * 8704, 32, 8, 128, 512) == 0
+    one_long = (1, 512, 32768 + 512, 32, 8, 128, 512)
+    need = lib.msgl_paged_prefill_workspace_bytes(*one_long)
+    assert need > 0 and need % (512 * 32 * (128 + 1) * 4) == 0
+    assert lib.msgl_set_tuning(6, 1) == 0
+    assert lib.msgl_paged_prefill_workspace_bytes(*one_long) == 0
+    assert lib.msgl_set_tuning(6, 0) == 0
+    # state pool: size checks come before any pointer is touched; nothing to do is not an error
+    def slots(slot_stride=64, row=64, layers=2, num_slots=4, layer_stride=256, pairs=1, slab=fake, dst=fake):
+        return lib.msgl_copy_state_slots(slab, layer_stride, slot_stride, row, layers, num_slots, None,
+                                         dst, pairs, None)
+    assert slots(slot_stride=32) == -9
+    assert slots(layer_stride=128) == -9
+    assert slots(pairs=-1) == -9
+    assert slots(pairs=0) == 0 and slots(layers=0) == 0 and slots(row=0, slot_stride=0, layer_stride=0) == 0
+    assert slots(slab=None) == -1 and slots(dst=None) == -1
 
 
 def _t(shape, dtype=torch.bfloat16):
