@@ -101,3 +101,37 @@ def test_benchmark_shapes_repeat_bit_identical(gpu, cfg, variant, head_dim):
                            sliding_window_size=g.sliding_window_size)
         torch.cuda.synchronize()
         assert torch.equal(out.cpu().view(torch.int16), first), f"run {i} differs from run 0"
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_extend_shapes_repeat_bit_identical(gpu, seed):
+    """Random ragged extends (both head sizes, every mask, forced key splits on half of them), each
+    launched 12 times: a race that needs an unusual shape still has to show as a changed bit."""
+    import random
+
+    from test_gpu_fuzz import HEADS, _length
+
+    rng = random.Random(7000 + seed)
+    n_q, n_kv = rng.choice(HEADS)
+    d = rng.choice([128, 256])
+    batch = rng.randrange(1, 7)
+    ext = [max(1, _length(rng, 400)) for _ in range(batch)]
+    kv = [e + (_length(rng, 3000) if rng.random() < 0.8 else 0) for e in ext]
+    is_cross = rng.random() < 0.3
+    window = rng.choice([0, 0, 17, 100, 1000])
+    splits = rng.choice([0, 0, 2, 5, 32])
+    wl = build_workload("t", "prefill", seed=seed, n_q=n_q, n_kv=n_kv, head_dim=d, kv_lens=kv,
+                        extend_lens=ext, pool_factor=1.2, is_cross_attention=is_cross,
+                        sliding_window_size=window)
+    g = wl.to(gpu)
+    print(f"repeat random seed={seed} heads={n_q}/{n_kv} d={d} ext={ext} kv={kv} cross={is_cross} "
+          f"W={window} key_splits={splits}", flush=True)
+    _lib.set_tuning(_lib.TUNE_PREFILL_KEY_SPLITS, splits)
+    try:
+        outs = [_prefill(g, max(ext), is_cross_attention=is_cross, sliding_window_size=window)
+                for _ in range(12)]
+        torch.cuda.synchronize()
+    finally:
+        _lib.set_tuning(_lib.TUNE_PREFILL_KEY_SPLITS, 0)
+    for i, out in enumerate(outs[1:], 1):
+        assert torch.equal(out.view(torch.int16), outs[0].view(torch.int16)), f"run {i} differs from run 0"
