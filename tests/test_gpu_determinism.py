@@ -135,3 +135,40 @@ def test_random_extend_shapes_repeat_bit_identical(gpu, seed):
         _lib.set_tuning(_lib.TUNE_PREFILL_KEY_SPLITS, 0)
     for i, out in enumerate(outs[1:], 1):
         assert torch.equal(out.view(torch.int16), outs[0].view(torch.int16)), f"run {i} differs from run 0"
+
+
+@pytest.mark.parametrize("seed", range(30))
+def test_random_decode_and_verify_shapes_repeat_bit_identical(gpu, seed):
+    """The split-K kernel and its merge on random batches (empty and one-token requests, several
+    requests per segment, one request over many segments), decode and short query blocks."""
+    import random
+
+    from test_gpu_fuzz import HEADS, _length
+
+    rng = random.Random(8000 + seed)
+    n_q, n_kv = rng.choice([h for h in HEADS if h[0] // h[1] <= 16])
+    d = rng.choice([128, 256])
+    batch = rng.randrange(1, 40)
+    q_len = rng.choice([0, 0, 1, 2, 3, 8])  # 0: decode
+    q_len = min(q_len, 64 // (n_q // n_kv))
+    hi = rng.choice([40, 300, 5000])
+    lens = [_length(rng, hi) for _ in range(batch)]
+    if q_len == 0:
+        lens = [max(n, 1) if i == 0 else n for i, n in enumerate(lens)]
+        wl = build_workload("t", "decode", seed=seed, n_q=n_q, n_kv=n_kv, head_dim=d, kv_lens=lens,
+                            pool_factor=1.2)
+        g = wl.to(gpu)
+        run = lambda: paged_decode_attention(g.q, g.k_cache, g.v_cache, g.kv_indptr, g.kv_indices,
+                                             g.num_kv_splits, g.sm_scale, g.max_kv_splits)
+    else:
+        window = rng.choice([0, 0, 64, 1000])
+        wl = build_workload("t", "prefill", seed=seed, n_q=n_q, n_kv=n_kv, head_dim=d,
+                            kv_lens=[n + q_len for n in lens], extend_lens=[q_len] * batch,
+                            pool_factor=1.2, sliding_window_size=window)
+        g = wl.to(gpu)
+        run = lambda: _prefill(g, q_len, sliding_window_size=window)
+    print(f"repeat random split-K seed={seed} heads={n_q}/{n_kv} d={d} q_len={q_len} lens={lens}", flush=True)
+    outs = [run() for _ in range(12)]
+    torch.cuda.synchronize()
+    for i, out in enumerate(outs[1:], 1):
+        assert torch.equal(out.view(torch.int16), outs[0].view(torch.int16)), f"run {i} differs from run 0"
