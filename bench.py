@@ -538,8 +538,8 @@ def run_radix_cache(cpu_baseline: bool):
 
 def run_small_launch_extends(dev, steps: int, warmup: int):
     """Extends too small to fill the chip (one long request, a short chunk): the tile kernels with
-    their keys in one pass (knob 1) against the library's own choice of key splits.  Not a BASELINE
-    shape; shows what the split buys and that both give the same result."""
+    their keys in one pass (knob 1) against the library's own choice of key splits.  Not one of the
+    benchmark shapes; shows what the split buys and that both give the same result."""
     import torch
 
     from mini_sglang_amd.workloads import build_workload

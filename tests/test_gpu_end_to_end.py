@@ -96,10 +96,10 @@ def test_prefix_reuse_extend_and_decode(gpu):
     toks = lambda n: rng.integers(0, VOCAB, size=n).tolist()
     seq_a, seq_b = toks(150), toks(70)
 
-    # ---- round 1: two fresh requests, prefilled together, then handed to the radix cache ----
+    # ---- first batch: two fresh requests, prefilled together, then handed to the radix cache ----
     for row, seq in ((0, seq_a), (1, seq_b)):
         layer.page_table[row, :len(seq)] = layer.allocate(len(seq)).to(gpu)
-    print("end to end: round 1", flush=True)
+    print("end to end: first batch", flush=True)
     out1, _ = layer.extend([(0, seq_a, 0), (1, seq_b, 0)])
     assert_close_bf16(out1[:150], layer.dense_reference(seq_a, list(range(150))), "request A")
     assert_close_bf16(out1[150:], layer.dense_reference(seq_b, list(range(70))), "request B")
@@ -107,7 +107,7 @@ def test_prefix_reuse_extend_and_decode(gpu):
         ids = torch.tensor(seq, dtype=torch.int32)
         assert layer.radix.insert_prefix(ids, layer.page_table[row, :len(seq)].cpu()) == 0
 
-    # ---- round 2: C shares 97 tokens with A, D shares all of B and goes on --------------------
+    # ---- second batch: C shares 97 tokens with A, D shares all of B and goes on --------------------
     seq_c = seq_a[:97] + toks(45)
     seq_d = seq_b + toks(30)
     plan = []
@@ -121,7 +121,7 @@ def test_prefix_reuse_extend_and_decode(gpu):
         plan.append((row, seq, n, handle))
     assert [p[2] for p in plan] == [97, 70]
     assert layer.radix.size_info.protected_size == 97 + 70
-    print("end to end: round 2 (cached prefixes 97 and 70)", flush=True)
+    print("end to end: second batch (cached prefixes 97 and 70)", flush=True)
     out2, _ = layer.extend([(row, seq, n) for row, seq, n, _ in plan])
     assert_close_bf16(out2[:45], layer.dense_reference(seq_c, list(range(97, 142))), "request C on A's prefix")
     assert_close_bf16(out2[45:], layer.dense_reference(seq_d, list(range(70, 100))), "request D on B's prefix")
