@@ -172,3 +172,37 @@ def test_random_decode_and_verify_shapes_repeat_bit_identical(gpu, seed):
     torch.cuda.synchronize()
     for i, out in enumerate(outs[1:], 1):
         assert torch.equal(out.view(torch.int16), outs[0].view(torch.int16)), f"run {i} differs from run 0"
+
+
+@pytest.mark.parametrize("head_dim", [128, 256])
+@pytest.mark.parametrize("kind", ["extend", "extend_split", "verify", "decode"])
+def test_repeat_bit_identical_while_another_stream_saturates_memory(gpu, head_dim, kind):
+    """Large device copies on a second stream change when loads return and how far waves drift
+    apart; the results must not notice."""
+    if kind == "decode":
+        wl = build_workload("t", "decode", seed=940, n_q=32, n_kv=8, head_dim=head_dim,
+                            kv_lens=[3000, 17, 900, 4000, 64, 2500, 129, 7000], pool_factor=1.1)
+        g = wl.to(gpu)
+        run = lambda: paged_decode_attention(g.q, g.k_cache, g.v_cache, g.kv_indptr, g.kv_indices,
+                                             g.num_kv_splits, g.sm_scale, g.max_kv_splits)
+    else:
+        ext = {"extend": [300, 70, 513], "extend_split": [300], "verify": [6, 6, 6, 6]}[kind]
+        pre = {"extend": [3000, 0, 700], "extend_split": [20000], "verify": [3000, 17, 900, 4000]}[kind]
+        wl = build_workload("t", "prefill", seed=941, n_q=16, n_kv=4, head_dim=head_dim,
+                            kv_lens=[p + e for p, e in zip(pre, ext)], extend_lens=ext, pool_factor=1.1)
+        g = wl.to(gpu)
+        run = lambda: _prefill(g, max(ext))
+    print(f"repeat under contention head_dim={head_dim} {kind}", flush=True)
+    quiet = run()
+    torch.cuda.synchronize()
+    src = torch.empty(256 << 20, dtype=torch.uint8, device=gpu)
+    dst = torch.empty_like(src)
+    side = torch.cuda.Stream(device=gpu)
+    side.wait_stream(torch.cuda.current_stream(gpu))
+    with torch.cuda.stream(side):
+        for _ in range(40):
+            dst.copy_(src, non_blocking=True)
+    outs = [run() for _ in range(25)]
+    torch.cuda.synchronize()
+    for i, out in enumerate(outs):
+        assert torch.equal(out.view(torch.int16), quiet.view(torch.int16)), f"run {i} differs"
