@@ -725,7 +725,12 @@ def main():
             "parity_ok": pre.get("parity_ok"), "kv_pool_bit_exact": pre.get("kv_pool_bit_exact"),
         }
         if not args.no_mfma_probe:
-            result["prefill"]["mfma_rate_probe"] = mfma_rate_probe()
+            probe = mfma_rate_probe()
+            result["prefill"]["mfma_rate_probe"] = probe
+            if probe and probe.get("random_operands"):
+                # the same MFMA instruction issued back to back on random operands, on this box,
+                # now: what the board sustains under its power limit
+                result["prefill"]["frac_of_measured_mfma_rate"] = pre["achieved_TFLOPs"] / probe["random_operands"]
     if not args.no_metadata:
         result["qk_norm_rope_store"] = run_norm_rope_store(dev, args.steps, args.warmup,
                                                            not args.no_cpu_baseline)
