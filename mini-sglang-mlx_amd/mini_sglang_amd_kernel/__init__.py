@@ -31,10 +31,37 @@ def _fail(op: str, msg: str):
     raise RuntimeError(f"{op}: {msg}")
 
 
+_raw_current_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream_ptr(stream, device) -> int:
-    if stream is None:
-        stream = torch.cuda.current_stream(device)
-    return int(stream.cuda_stream)
+    if stream is not None:
+        return int(stream.cuda_stream)
+    if _raw_current_stream is not None:  # the handle without building a Stream object
+        return int(_raw_current_stream(device.index if device.index is not None
+                                       else torch.cuda.current_device()))
+    return int(torch.cuda.current_stream(device).cuda_stream)
+
+
+class _on_device:
+    """``torch.cuda.device(dev)`` that costs nothing when ``dev`` is current already (the usual
+    case: one process per GPU)."""
+
+    __slots__ = ("_guard",)
+
+    def __init__(self, dev: torch.device):
+        index = dev.index
+        self._guard = None if index is None or index == torch.cuda.current_device() \
+            else torch.cuda.device(dev)
+
+    def __enter__(self):
+        if self._guard is not None:
+            self._guard.__enter__()
+
+    def __exit__(self, *exc):
+        if self._guard is not None:
+            self._guard.__exit__(*exc)
+        return False
 
 
 def _require_device(op: str, *tensors: torch.Tensor) -> torch.device:
@@ -106,7 +133,7 @@ def store_kv_cache(k_cache: torch.Tensor, v_cache: torch.Tensor, indices: torch.
     k, k_stride0 = _src(k)
     v, v_stride0 = _src(v)
     indices = indices if indices.is_contiguous() else indices.contiguous()
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         rc = _lib.load().msgl_store_kv_cache(
             k_cache.data_ptr(), v_cache.data_ptr(), indices.data_ptr(), k.data_ptr(),
             v.data_ptr(), length, num_kv_heads, head_dim, num_pages,
@@ -182,7 +209,7 @@ def paged_decode_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torc
         return out
     lib = _lib.load()
     total_kv = kv_indices.shape[0]
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         ws_bytes = lib.msgl_paged_decode_workspace_bytes(batch, total_kv, num_q_heads,
                                                          num_kv_heads, head_dim)
         ws = _workspace(ws_bytes, dev, stream)
@@ -249,7 +276,7 @@ def paged_prefill_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
         return out
     lib = _lib.load()
     total_kv = kv_indices.shape[0]
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         ws_bytes = lib.msgl_paged_prefill_workspace_bytes(
             batch, total_q, total_kv, num_q_heads, num_kv_heads, head_dim, int(max_len_extend))
         ws = _workspace(ws_bytes, dev, stream)
