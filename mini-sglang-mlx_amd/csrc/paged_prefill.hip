@@ -110,6 +110,10 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
   const int row0 = qblk * kRows;
   if (row0 >= rows_total) return;
 
+  // A wave all of whose rows lie past the end of the request's rows (possible in its last query
+  // block) takes part in moving tiles and in every barrier but computes nothing: its SIMD's
+  // matrix pipe is left to the wave that shares it.
+  const bool idle = __builtin_amdgcn_readfirstlane(row0 + w * RT * 32 >= rows_total ? 1 : 0) != 0;
   const int qi_lo = row0 / p.group;
   const int qi_hi = min(rows_total - 1, row0 + kRows - 1) / p.group;
   int k_hi = p.is_cross ? kn : min(kn, prefix + qi_hi + 1);
@@ -453,70 +457,91 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
     slot_load(k_lo + 2 * kBN);
     wait_all_vm();
     __syncthreads();
-    Scores sa, sb;
-    Stats st_a, st_b;
-    bf16x8_t pb_a[RT][2], pb_b[RT][2];
-    qk_half(0, 0, sa);
-    st_a.mul = p.scale_log2e;
-    if (needs_mask(k_lo)) {
-      mask_in_place(sa, k_lo);
-      st_a.mul = 1.0f;
-    }
-    {
-      float mx[RT];
-      lane_max(sa, mx);
-      decide(mx, st_a);
-    }
-    st_b.mul = 1.0f;
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt) {
-      st_b.alpha[rt] = 1.0f;
-      st_b.m_safe[rt] = 0.f;
-#pragma unroll
-      for (int u = 0; u < 2; ++u) pb_b[rt][u] = as_bf16x8(u32x4_t{0u, 0u, 0u, 0u});
-    }
     // byte offsets of the stages: K of tiles j, j+1 and the one being filled; V of tiles
     // j-1, j and the one being filled (the first P is zero, so "tile -1" may alias tile 0)
     uint32_t k_cur = 0, k_next = kKStage, k_fill = 2 * kKStage;
     uint32_t v_prev = kVBase, v_cur = kVBase, v_fill = kVBase + kVStage, v_spare = kVBase + 2 * kVStage;
-    bf16x8_t kops[4];
+    if (idle) {
+      // the same moves, waits and barriers as the computing waves, tile by tile
+      for (int j = 0; j < n_tiles; ++j) {
+        offsets_from_slots();
+        slot_load(k_lo + (j + 3) * kBN);
 #pragma unroll
-    for (int e = 0; e < 4; ++e) kops[e] = k_operand(smem + k_cur + k_lane + 512, e);
-    for (int j = 0; j < n_tiles; ++j) {
-      const int tb = k_lo + j * kBN;
-      // the moves of this iteration (V of tile j+1, K of tile j+2) are issued one per slice
-      // of the first half, between its MFMAs; the slot ids of tile j+3 are requested now and
-      // used in the next iteration
-      offsets_from_slots();
-      slot_load(tb + 3 * kBN);
-      // half (j,0): scores of (j,1) from K of tile j, P V of (j-1,1) from V of tile j-1
+        for (int n = 0; n < 2 * UPW; ++n) move(n, k_fill, v_fill);
+        rotate_v_offsets();
+        wait_all_vm();
+        __syncthreads();
+        const uint32_t k_freed = k_cur;
+        k_cur = k_next;
+        k_next = k_fill;
+        k_fill = k_freed;
+        const uint32_t v_freed = (j == 0) ? v_spare : v_prev;
+        v_prev = v_cur;
+        v_cur = v_fill;
+        v_fill = v_freed;
+      }
+    } else {
+      Scores sa, sb;
+      Stats st_a, st_b;
+      bf16x8_t pb_a[RT][2], pb_b[RT][2];
+      qk_half(0, 0, sa);
+      st_a.mul = p.scale_log2e;
+      if (needs_mask(k_lo)) {
+        mask_in_place(sa, k_lo);
+        st_a.mul = 1.0f;
+      }
+      {
+        float mx[RT];
+        lane_max(sa, mx);
+        decide(mx, st_a);
+      }
+      st_b.mul = 1.0f;
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        st_b.alpha[rt] = 1.0f;
+        st_b.m_safe[rt] = 0.f;
+#pragma unroll
+        for (int u = 0; u < 2; ++u) pb_b[rt][u] = as_bf16x8(u32x4_t{0u, 0u, 0u, 0u});
+      }
+      bf16x8_t kops[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) kops[e] = k_operand(smem + k_cur + k_lane + 512, e);
+      for (int j = 0; j < n_tiles; ++j) {
+        const int tb = k_lo + j * kBN;
+        // the moves of this iteration (V of tile j+1, K of tile j+2) are issued one per slice
+        // of the first half, between its MFMAs; the slot ids of tile j+3 are requested now and
+        // used in the next iteration
+        offsets_from_slots();
+        slot_load(tb + 3 * kBN);
+        // half (j,0): scores of (j,1) from K of tile j, P V of (j-1,1) from V of tile j-1
+        rescale(st_b.alpha);
+        fused_half(sa, st_a, sb, st_b, needs_mask(tb + 32), tb + 32, smem + k_cur + k_lane + 512,
+                   smem + v_prev + v_lane + 512, smem + k_next + k_lane, kops, pb_b, pb_a,
+                   [&](int sl) {
+                     constexpr int PER = 2 * UPW / 4;
+#pragma unroll
+                     for (int n = sl * PER; n < (sl + 1) * PER; ++n) move(n, k_fill, v_fill);
+                   });
+        rotate_v_offsets();
+        // half (j,1): scores of (j+1,0) from K of tile j+1, P V of (j,0) from V of tile j
+        rescale(st_a.alpha);
+        fused_half(sb, st_b, sa, st_a, needs_mask(tb + 64), tb + 64, smem + k_next + k_lane,
+                   smem + v_cur + v_lane, smem + k_next + k_lane + 512, kops, pb_a, pb_b, [](int) {});
+        wait_all_vm();
+        __syncthreads();
+        const uint32_t k_freed = k_cur;
+        k_cur = k_next;
+        k_next = k_fill;
+        k_fill = k_freed;
+        const uint32_t v_freed = (j == 0) ? v_spare : v_prev;
+        v_prev = v_cur;
+        v_cur = v_fill;
+        v_fill = v_freed;
+      }
+      // the last half's P V is still owed
       rescale(st_b.alpha);
-      fused_half(sa, st_a, sb, st_b, needs_mask(tb + 32), tb + 32, smem + k_cur + k_lane + 512,
-                 smem + v_prev + v_lane + 512, smem + k_next + k_lane, kops, pb_b, pb_a,
-                 [&](int sl) {
-                   constexpr int PER = 2 * UPW / 4;
-#pragma unroll
-                   for (int n = sl * PER; n < (sl + 1) * PER; ++n) move(n, k_fill, v_fill);
-                 });
-      rotate_v_offsets();
-      // half (j,1): scores of (j+1,0) from K of tile j+1, P V of (j,0) from V of tile j
-      rescale(st_a.alpha);
-      fused_half(sb, st_b, sa, st_a, needs_mask(tb + 64), tb + 64, smem + k_next + k_lane,
-                 smem + v_cur + v_lane, smem + k_next + k_lane + 512, kops, pb_a, pb_b, [](int) {});
-      wait_all_vm();
-      __syncthreads();
-      const uint32_t k_freed = k_cur;
-      k_cur = k_next;
-      k_next = k_fill;
-      k_fill = k_freed;
-      const uint32_t v_freed = (j == 0) ? v_spare : v_prev;
-      v_prev = v_cur;
-      v_cur = v_fill;
-      v_fill = v_freed;
+      pv_half(v_prev, 1, pb_b);
     }
-    // the last half's P V is still owed
-    rescale(st_b.alpha);
-    pv_half(v_prev, 1, pb_b);
     __syncthreads();  // the epilogue reuses the stages as its output staging area
   }
 

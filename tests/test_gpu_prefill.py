@@ -420,3 +420,22 @@ def test_one_long_request_splits_its_keys_by_itself(gpu, head_dim, extend):
     wl = build_workload("t", "prefill", seed=760 + extend, n_q=n_q, n_kv=n_kv, head_dim=head_dim,
                         kv_lens=[prefix + extend], extend_lens=[extend], pool_factor=1.1, store_new=True)
     _check(wl, gpu, f"one long request head_dim={head_dim} extend={extend}")
+
+
+@pytest.mark.parametrize("head_dim", [128, 256])
+def test_partially_filled_query_blocks_idle_waves(gpu, head_dim):
+    """Last query blocks with 1 .. 7 of the eight waves' row ranges empty (head_dim 128: such waves
+    move tiles and pass barriers but compute nothing), next to full blocks, on prefixes long enough
+    for many tiles; the smallest-query route is kept off so that every request takes a tile kernel."""
+    from mini_sglang_amd_kernel import _lib
+
+    # group 4: an extend of e tokens has 4 e rows; blocks hold 256 (head_dim 128) or 128 rows
+    ext = [17, 24, 33, 41, 49, 57, 64, 65, 72, 100, 121]
+    wl = build_workload("t", "prefill", seed=960, n_q=8, n_kv=2, head_dim=head_dim,
+                        kv_lens=[700 + 37 * i + e for i, e in enumerate(ext)], extend_lens=ext,
+                        pool_factor=1.2, store_new=True)
+    _lib.set_tuning(_lib.TUNE_SMALLQ_MAXCOLS, -1)
+    try:
+        _check(wl, gpu, f"partially filled query blocks head_dim={head_dim}")
+    finally:
+        _lib.set_tuning(_lib.TUNE_SMALLQ_MAXCOLS, 0)
