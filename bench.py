@@ -34,6 +34,7 @@ for _p in (ROOT, os.path.join(ROOT, "mini-sglang-mlx_amd")):
 METRIC = "decode attn HBM TB/s (% of peak) + chunked-prefill attn TFLOP/s (% MFMA peak)"
 HBM_PEAK = 8.0e12
 MFMA_PEAK = 2.5e15
+SPINUP_MS = 100.0  # untimed run of the step before its warm-up steps (clock settling)
 
 
 def log(*a):
@@ -41,25 +42,42 @@ def log(*a):
 
 
 def time_steps(fn, steps: int, warmup: int):
-    """Time exactly `steps` back-to-back steps between two HIP events recorded on torch's
-    current stream (the stream every operator launches on), bracketed by device syncs.
-    A second pass brackets every step with its own event pair for the min / median; those
-    figures carry the event markers' own few microseconds."""
+    """`warmup` untimed steps, then exactly `steps` back-to-back steps between two HIP events
+    recorded on torch's current stream (the stream every operator launches on), bracketed by
+    device syncs: that mean is the reported figure.  Two diagnostic passes follow: one that
+    brackets every step with its own event pair (min / median / the per-step list; those carry
+    the event markers' own few microseconds), and a repeat of the first pass, which shows
+    whether the first one still saw the clocks settling."""
     import torch
 
+    def loop_ms():
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        e0.record()
+        for _ in range(steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1), (time.perf_counter() - t0) * 1e3
+
+    # The shader clock needs some tens of milliseconds of load to settle (measured: the MFMA
+    # kernels keep getting faster for the first ~30 ms after an idle spell), so the step first
+    # runs untimed for SPINUP_MS of device time; the `warmup` steps the caller asked for follow.
+    spin0 = torch.cuda.Event(enable_timing=True)
+    spin0.record()
+    while True:
+        for _ in range(4):
+            fn()
+        spin1 = torch.cuda.Event(enable_timing=True)
+        spin1.record()
+        spin1.synchronize()
+        if spin0.elapsed_time(spin1) >= SPINUP_MS:
+            break
     for _ in range(warmup):
         fn()
-    torch.cuda.synchronize()
-    e0 = torch.cuda.Event(enable_timing=True)
-    e1 = torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    e0.record()
-    for _ in range(steps):
-        fn()
-    e1.record()
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3
-    loop_ms = e0.elapsed_time(e1)
+    loop, wall_ms = loop_ms()
     starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
     ends = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
     for i in range(steps):
@@ -68,7 +86,9 @@ def time_steps(fn, steps: int, warmup: int):
         ends[i].record()
     torch.cuda.synchronize()
     per = [s.elapsed_time(e) for s, e in zip(starts, ends)]
-    return loop_ms / steps, per, wall_ms
+    again, _ = loop_ms()
+    time_steps.last_repeat_ms = again / steps
+    return loop / steps, per, wall_ms
 
 
 def make_step(g):
@@ -156,6 +176,8 @@ def run_config(cfg: int, variant: str, steps: int, warmup: int, check: bool, cpu
         "total_kv_tokens": int(sum(wl.kv_lens)), "total_q_tokens": int(sum(wl.extend_lens)),
         "sliding_window": wl.sliding_window_size,
         "ms_mean": mean_ms, "ms_median": med_ms, "ms_min": min(per),
+        "ms_mean_repeat": time_steps.last_repeat_ms, "spinup_ms": SPINUP_MS,
+        "per_step_us": [round(x * 1e3, 1) for x in per],
         "wall_ms_per_step": wall_ms / steps, "steps": steps, "warmup": warmup,
         "algorithmic_bytes": abytes, "algorithmic_flops": aflops, "store_bytes": sbytes,
         "bound": bound, "gen_s": round(gen_s, 1),
@@ -564,12 +586,10 @@ def run_small_launch_extends(dev, steps: int, warmup: int):
         outs = {}
         for label, knob in (("one_pass", 1), ("key_split", 0)):
             _lib.set_tuning(_lib.TUNE_PREFILL_KEY_SPLITS, knob)
-            try:
-                ms, _, _ = time_steps(step, max(3, steps // 5), max(1, warmup // 5))
-                outs[label] = step().float()
-                torch.cuda.synchronize()
-            finally:
-                _lib.set_tuning(_lib.TUNE_PREFILL_KEY_SPLITS, 0)
+            ms, _, _ = time_steps(step, max(3, steps // 5), max(1, warmup // 5))
+            outs[label] = step().float()
+            torch.cuda.synchronize()
+            _lib.set_tuning(_lib.TUNE_PREFILL_KEY_SPLITS, 0)
             row[label + "_us"] = ms * 1e3
             row[label + "_TFLOPs"] = row["algorithmic_flops"] / (ms * 1e-3) / 1e12
         row["max_abs_diff"] = float((outs["one_pass"] - outs["key_split"]).abs().max())
@@ -581,18 +601,60 @@ def run_small_launch_extends(dev, steps: int, warmup: int):
     return rows
 
 
+PROBE_SRC = os.path.join(ROOT, "bench_probes.hip")
+PROBE_LIB = os.path.join(ROOT, "bench_probes.so")
+
+
+def build_probes(force: bool = False) -> str:
+    """Compile bench_probes.hip (the two measurement aids below) into bench_probes.so beside this
+    file.  hipcc cross-compiles for gfx950, so this also runs where there is no GPU."""
+    import subprocess
+
+    if force or not os.path.exists(PROBE_LIB) or os.path.getmtime(PROBE_SRC) > os.path.getmtime(PROBE_LIB):
+        cmd = [os.environ.get("HIPCC", "/opt/rocm/bin/hipcc"), "--offload-arch=gfx950", "-O3",
+               "-std=c++17", "-fPIC", "-fvisibility=hidden", "-Xclang", "-target-feature", "-Xclang",
+               "-packed-fp32-ops", "-shared", PROBE_SRC, "-o", PROBE_LIB]
+        proc = subprocess.run(cmd, capture_output=True, text=True)
+        if proc.returncode != 0:
+            raise RuntimeError(f"hipcc failed for bench_probes.hip:\n{proc.stderr}")
+    return PROBE_LIB
+
+
+def _probe_lib():
+    import ctypes
+
+    return ctypes.CDLL(build_probes())
+
+
+def hbm_read_probe(gib: int = 4, reps: int = 5):
+    """A plain streaming read of `gib` GiB (16 bytes per lane and load, consecutive lanes on
+    consecutive addresses, far beyond the 256 MB Infinity Cache): the rate the memory system
+    gives a kernel that does nothing but read, beside the datasheet's 8 TB/s."""
+    import ctypes
+
+    lib = _probe_lib()
+    lib.msgl_probe_hbm_read.restype = ctypes.c_int
+    lib.msgl_probe_hbm_read.argtypes = [ctypes.c_size_t, ctypes.c_int, ctypes.POINTER(ctypes.c_double),
+                                        ctypes.POINTER(ctypes.c_double)]
+    best, mean = ctypes.c_double(0), ctypes.c_double(0)
+    rc = lib.msgl_probe_hbm_read(gib << 30, reps, ctypes.byref(best), ctypes.byref(mean))
+    if rc != 0:
+        return None
+    log(f"[hbm read probe] {gib} GiB x {reps}: best {best.value:.3f} TB/s, mean {mean.value:.3f} TB/s")
+    return {"unit": "TB/s", "bytes": gib << 30, "reps": reps, "best": best.value, "mean": mean.value,
+            "frac_of_datasheet_peak": mean.value * 1e12 / HBM_PEAK,
+            "kernel": "grid-stride read, 16 B per lane and load, 8 loads in flight per lane"}
+
+
 def mfma_rate_probe():
     """Sustained v_mfma_f32_32x32x16_bf16 rate of the whole chip on register-resident operands,
     nothing else running: all-zero operands and N(0,1) operands that change every instruction.
     The board lowers its shader clock to hold its power limit and MFMA power grows with the
-    number of toggling operand bits, so the second figure, not the datasheet peak, is what a
-    kernel on random bf16 data can reach."""
+    number of toggling operand bits, so the second figure is context for the prefill number;
+    `roofline.frac` stays the fraction of the datasheet peak."""
     import ctypes
 
-    path = os.path.join(ROOT, "mini-sglang-mlx_amd", "lib", "libmsgl_probes.so")
-    if not os.path.exists(path):
-        return None
-    lib = ctypes.CDLL(path)
+    lib = _probe_lib()
     lib.msgl_probe_mfma_rate.restype = ctypes.c_int
     lib.msgl_probe_mfma_rate.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_double),
                                          ctypes.POINTER(ctypes.c_double)]
@@ -625,9 +687,8 @@ def main():
                     help="skip the figures of the kernels either side of the path: on-device metadata "
                          "build (slot table -> CSR arrays) and fused q/k norm + rope + KV-store")
     ap.add_argument("--no-mfma-probe", action="store_true",
-                    help="skip the measurement of the matrix pipe's sustained rate on zero and "
-                         "on random operands (the power-limited ceiling the prefill figure is "
-                         "reported beside)")
+                    help="skip the two measurement aids: the matrix pipe's sustained rate on zero "
+                         "and on random operands, and the rate of a plain streaming read of 4 GiB")
     ap.add_argument("--cpu-flops", type=float, default=3e11,
                     help="flop budget of the CPU baseline sample per shape")
     args = ap.parse_args()
@@ -731,6 +792,8 @@ def main():
                 # the same MFMA instruction issued back to back on random operands, on this box,
                 # now: what the board sustains under its power limit
                 result["prefill"]["frac_of_measured_mfma_rate"] = pre["achieved_TFLOPs"] / probe["random_operands"]
+    if not args.no_mfma_probe:
+        result["hbm_read_probe"] = hbm_read_probe()
     if not args.no_metadata:
         result["qk_norm_rope_store"] = run_norm_rope_store(dev, args.steps, args.warmup,
                                                            not args.no_cpu_baseline)

@@ -1,10 +1,18 @@
-// What the matrix pipe sustains on this board when nothing else runs: back-to-back
+// Two measurements that bench.py reports beside the attention figures; benchmarking aids, built
+// into bench_probes.so beside bench.py, not part of the paged-attention library.
+//
+// (1) What the matrix pipe sustains on this board when nothing else runs: back-to-back
 // v_mfma_f32_32x32x16_bf16 on register-resident operands, one workgroup of four waves per CU.
 // The board holds a power limit by lowering the shader clock, and MFMA power depends on how
 // many operand bits toggle, so the rate is measured for all-zero operands and for operands
 // drawn from N(0,1) that change with every instruction.  The second figure is the ceiling a
 // bf16 attention kernel on random data is measured against; the datasheet peak assumes the
-// boost clock.  Benchmarking aid only: not part of the paged-attention library.
+// boost clock.
+//
+// (2) What a plain streaming read sustains: every lane reads 16 bytes per load, consecutive
+// lanes consecutive addresses, a grid-stride loop over a buffer far larger than the 256 MB
+// Infinity Cache, eight loads in flight per lane.  The HBM-bound attention kernels are read
+// beside this figure as well as beside the datasheet's 8 TB/s.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -63,7 +71,76 @@ __global__ __launch_bounds__(256) void mfma_rate_kernel(int random_operands, int
   }
 }
 
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
+__global__ __launch_bounds__(256) void hbm_read_kernel(const u32x4_t* __restrict__ src, size_t n_vec,
+                                                       uint32_t* sink) {
+  const size_t stride = (size_t)gridDim.x * 256;
+  size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  u32x4_t acc = {0u, 0u, 0u, 0u};
+  for (; i + 7 * stride < n_vec; i += 8 * stride) {
+    u32x4_t v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = __builtin_nontemporal_load(src + i + u * stride);
+#pragma unroll
+    for (int u = 0; u < 8; ++u) acc ^= v[u];
+  }
+  for (; i < n_vec; i += stride) acc ^= __builtin_nontemporal_load(src + i);
+  const uint32_t x = acc[0] ^ acc[1] ^ acc[2] ^ acc[3];
+  if (x == 0x9e3779b9u) sink[0] = x;  // never true for the fill pattern; keeps the loads alive
+}
+
 }  // namespace
+
+// Reads `bytes` (a multiple of 16; at least 1 GiB is sensible) `reps` times and reports the best
+// and the mean rate in TB/s.  Blocking; allocates and frees its own buffer.  Returns 0 or a
+// hipError_t value.
+extern "C" __attribute__((visibility("default"))) int msgl_probe_hbm_read(size_t bytes, int reps,
+                                                                        double* best_tbps,
+                                                                        double* mean_tbps) {
+  int dev = 0, cus = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+  if (e != hipSuccess) return (int)e;
+  if (reps < 1 || bytes < 16) return (int)hipErrorInvalidValue;
+  void* buf = nullptr;
+  uint32_t* sink = nullptr;
+  e = hipMalloc(&buf, bytes);
+  if (e != hipSuccess) return (int)e;
+  e = hipMalloc(&sink, 4);
+  if (e != hipSuccess) {
+    (void)hipFree(buf);
+    return (int)e;
+  }
+  (void)hipMemset(buf, 0x5a, bytes);
+  const size_t n_vec = bytes / 16;
+  const dim3 grid((unsigned)(cus * 8)), block(256);
+  hipEvent_t t0, t1;
+  (void)hipEventCreate(&t0);
+  (void)hipEventCreate(&t1);
+  hipLaunchKernelGGL(hbm_read_kernel, grid, block, 0, 0, (const u32x4_t*)buf, n_vec, sink);
+  double best = 0.0, total_ms = 0.0;
+  for (int r = 0; r < reps; ++r) {
+    (void)hipEventRecord(t0, 0);
+    hipLaunchKernelGGL(hbm_read_kernel, grid, block, 0, 0, (const u32x4_t*)buf, n_vec, sink);
+    (void)hipEventRecord(t1, 0);
+    e = hipEventSynchronize(t1);
+    if (e != hipSuccess) break;
+    float ms = 0.f;
+    (void)hipEventElapsedTime(&ms, t0, t1);
+    total_ms += ms;
+    const double rate = (double)bytes / (ms * 1e-3) / 1e12;
+    if (rate > best) best = rate;
+  }
+  *best_tbps = best;
+  *mean_tbps = total_ms > 0.0 ? (double)bytes * reps / (total_ms * 1e-3) / 1e12 : 0.0;
+  (void)hipEventDestroy(t0);
+  (void)hipEventDestroy(t1);
+  (void)hipFree(buf);
+  (void)hipFree(sink);
+  return (int)e;
+}
 
 // Runs the probe on the current device (blocking).  tflops: achieved MFMA rate; shader_ghz:
 // shader clock during the run (cycle counter against the 100 MHz wall counter).

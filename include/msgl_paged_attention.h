@@ -235,8 +235,10 @@ MSGL_API int msgl_gdn_state_inplace(const void* q, const void* k, const void* v,
                            int64_t v_stride0, int32_t single_token_mode, void* stream);
 
 /*
- * Tuning knobs, for benchmarking only (0 = built-in heuristic).  Process-wide,
- * read at launch time; not part of the reference surface.
+ * Tuning knobs, for benchmarking only (0 = built-in heuristic).  One set per HOST THREAD
+ * (thread-local): msgl_set_tuning changes the calling thread's later calls only, so a
+ * *_workspace_bytes() call and the launch that follows it on the same thread agree whatever
+ * other threads set.  Read at launch time; not part of the reference surface.
  *   MSGL_TUNE_SEGMENTS       segments the split-K kernel cuts the visible token stream into
  *   MSGL_TUNE_MIN_SEGMENT    smallest segment length in tokens (multiple of 64)
  *   MSGL_TUNE_SMALLQ_MAXCOLS largest q_len*group routed to the split-K kernel

@@ -18,9 +18,6 @@ CSRC = os.path.join(HERE, "csrc")
 LIB_DIR = os.path.join(HERE, "lib")
 OBJ_DIR = os.path.join(HERE, "build")
 LIB_PATH = os.path.join(LIB_DIR, "libmsgl_paged_attention.so")
-# benchmarking aid (measured MFMA ceiling under the board's power limit); bench.py loads it
-PROBE_SRC = os.path.join(CSRC, "probes", "mfma_rate_probe.hip")
-PROBE_PATH = os.path.join(LIB_DIR, "libmsgl_probes.so")
 SOURCES = ["api.hip", "store_kv_cache.hip", "paged_splitkv.hip", "paged_prefill.hip", "paged_prefill_d256.hip",
            "build_metadata.hip", "qk_norm_rope_store.hip",
            "gdn_state.hip", "radix_cache.hip", "state_slots.hip"]
@@ -76,11 +73,6 @@ def build(force: bool = False, save_temps: bool = False) -> str:
         proc = subprocess.run(cmd, capture_output=True, text=True)
         if proc.returncode != 0:
             raise RuntimeError(f"link failed:\n{proc.stderr}")
-    if force or _newer([PROBE_SRC], PROBE_PATH):
-        cmd = [HIPCC, *FLAGS, "-shared", PROBE_SRC, "-o", PROBE_PATH]
-        proc = subprocess.run(cmd, capture_output=True, text=True)
-        if proc.returncode != 0:
-            raise RuntimeError(f"hipcc failed for the probe library:\n{proc.stderr}")
     return LIB_PATH
 
 

@@ -2,8 +2,6 @@
 // The checks mirror the reference's host functions (paged_decode_attention.cpp:25-62,
 // paged_prefill_attention.cpp:31-76, store_kv_cache.cpp:22-63) as far as raw pointers
 // and sizes can express them; rank and dtype-equality checks live in the Python shim.
-#include <atomic>
-
 #include <algorithm>
 
 #include "msgl_internal.h"
@@ -11,8 +9,11 @@
 
 namespace {
 
-std::atomic<int64_t> g_tune[3] = {{0}, {0}, {0}};
-std::atomic<int64_t> g_key_splits{0};
+// Benchmarking knobs live per host thread: the thread that sets one changes its own later
+// calls only, so a *_workspace_bytes() call and the launch that follows it on the same thread
+// always agree on the split, whatever other threads (one per stream) do.
+thread_local int64_t t_tune[3] = {0, 0, 0};
+thread_local int64_t t_key_splits = 0;
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
@@ -35,17 +36,17 @@ int check_common(const void* q, const void* k_cache, const void* v_cache, const 
 }
 
 int32_t min_segment() {
-  const int64_t t = g_tune[MSGL_TUNE_MIN_SEGMENT].load();
+  const int64_t t = t_tune[MSGL_TUNE_MIN_SEGMENT];
   if (t >= 64) return (int32_t)(t / 64 * 64);
   return msgl::kSplitKvMinSegment;
 }
 int32_t segments(int64_t total_kv, int64_t n_kv, int64_t head_dim, int64_t cols) {
-  const int64_t t = g_tune[MSGL_TUNE_SEGMENTS].load();
+  const int64_t t = t_tune[MSGL_TUNE_SEGMENTS];
   if (t >= 1) return (int32_t)(t < (1 << 20) ? t : (1 << 20));
   return msgl::splitkv_default_segments(total_kv, n_kv, head_dim, cols, min_segment());
 }
 int64_t smallq_max_cols() {
-  const int64_t t = g_tune[MSGL_TUNE_SMALLQ_MAXCOLS].load();
+  const int64_t t = t_tune[MSGL_TUNE_SMALLQ_MAXCOLS];
   if (t < 0) return 0;  // negative: never take the split-K route
   if (t > 0) return t < msgl::kSplitKvMaxCols ? t : msgl::kSplitKvMaxCols;
   return msgl::kSplitKvMaxCols;
@@ -91,11 +92,11 @@ int msgl_set_tuning(int32_t knob, int64_t value) {
     return MSGL_OK;
   }
   if (knob == MSGL_TUNE_PREFILL_KEY_SPLITS) {
-    g_key_splits.store(value < 0 ? 0 : value);
+    t_key_splits = value < 0 ? 0 : value;
     return MSGL_OK;
   }
   if (knob < 0 || knob > 2) return MSGL_ERR_SHAPE;
-  g_tune[knob].store(value);
+  t_tune[knob] = value;
   return MSGL_OK;
 }
 
@@ -111,7 +112,7 @@ int msgl_store_kv_cache(void* k_cache, void* v_cache, const int32_t* indices, co
     return MSGL_ERR_SHAPE;
   if (length == 0) return MSGL_OK;
   if (!k_cache || !v_cache || !indices || !k || !v) return MSGL_ERR_NULL_POINTER;
-  return msgl::launch_store_kv_cache(k_cache, v_cache, indices, k, v, length, row * elem_bytes,
+  return msgl::launch_store_kv_cache(k_cache, v_cache, indices, k, v, length, num_slots, row * elem_bytes,
                                      k_cache_stride0 * elem_bytes, v_cache_stride0 * elem_bytes,
                                      k_stride0 * elem_bytes, v_stride0 * elem_bytes,
                                      static_cast<hipStream_t>(stream));
@@ -201,7 +202,7 @@ size_t msgl_paged_prefill_workspace_bytes(int64_t batch, int64_t total_q, int64_
       // tile kernels: partials of a key split, if this launch would use one (a sliding window,
       // unknown here, can only lower the count)
       const int k = msgl::prefill_key_splits(batch, total_kv, num_kv_heads, group, max_len_extend, 0,
-                                             msgl::prefill_block_rows(head_dim), g_key_splits.load());
+                                             msgl::prefill_block_rows(head_dim), t_key_splits);
       return msgl::prefill_split_workspace_bytes(total_q, num_q_heads, head_dim, k);
     }
     const int32_t qc = chunk_queries(group);
@@ -300,7 +301,7 @@ int msgl_paged_prefill_attention(const void* q, const void* k_cache, const void*
   a.window = sliding_window_size;
   a.key_splits = msgl::prefill_key_splits(batch, total_kv, num_kv_heads, group, max_len_extend,
                                           sliding_window_size, msgl::prefill_block_rows(head_dim),
-                                          g_key_splits.load());
+                                          t_key_splits);
   if (a.key_splits > 1) {
     // the split is an optimisation: without room for its partials the keys go in one pass
     const size_t need = msgl::prefill_split_workspace_bytes(total_q, num_q_heads, head_dim, a.key_splits);
@@ -399,6 +400,7 @@ int msgl_qk_norm_rope_store(const void* q, const void* k, const void* v, int64_t
   a.kc_stride0 = k_cache_stride0;
   a.vc_stride0 = v_cache_stride0;
   a.n_tokens = n_tokens;
+  a.num_slots = num_slots;
   a.n_q = num_q_heads;
   a.n_kv = num_kv_heads;
   a.head_dim = head_dim;

@@ -174,8 +174,8 @@ __global__ __launch_bounds__(256) void gdn_state_kernel(GdnParams p) {
 
 }  // namespace
 
-static std::atomic<int> g_force_rows{0};
-void gdn_set_rows(int v) { g_force_rows.store(v == 1 || v == 2 || v == 4 ? v : 0); }
+static thread_local int t_force_rows = 0;  // benchmarking switch, one value per host thread
+void gdn_set_rows(int v) { t_force_rows = (v == 1 || v == 2 || v == 4) ? v : 0; }
 
 int launch_gdn_state(const GdnArgs& a, hipStream_t stream) {
   GdnParams p;
@@ -205,7 +205,7 @@ int launch_gdn_state(const GdnArgs& a, hipStream_t stream) {
   int r = 1;
   if (blocks_r1 >= 8 * 1024) r = 4;
   else if (blocks_r1 >= 4 * 1024) r = 2;
-  if (g_force_rows.load() > 0) r = g_force_rows.load();
+  if (t_force_rows > 0) r = t_force_rows;
   const int64_t blocks = heads * (kDV / (16 * r));
   if (blocks > 0x7fffffffLL) return MSGL_ERR_SHAPE;
   const dim3 grid((unsigned)blocks), block(256);

@@ -12,7 +12,7 @@ namespace msgl {
 
 // ---- store_kv_cache.hip ------------------------------------------------------------
 int launch_store_kv_cache(void* k_cache, void* v_cache, const int32_t* indices, const void* k,
-                          const void* v, int64_t length, int64_t row_bytes,
+                          const void* v, int64_t length, int64_t num_slots, int64_t row_bytes,
                           int64_t k_cache_stride_bytes, int64_t v_cache_stride_bytes,
                           int64_t k_stride_bytes, int64_t v_stride_bytes, hipStream_t stream);
 
@@ -113,7 +113,7 @@ struct NormRopeArgs {
   void* k_cache;
   void* v_cache;
   int64_t q_stride0, k_stride0, v_stride0, kc_stride0, vc_stride0;  // elements
-  int64_t n_tokens, n_q, n_kv, head_dim;
+  int64_t n_tokens, n_q, n_kv, head_dim, num_slots;
   float eps, rope_base;
 };
 int launch_qk_norm_rope_store(const NormRopeArgs& a, hipStream_t stream);

@@ -25,7 +25,6 @@
 //   boundary half tiles are scaled and masked in place before their softmax.
 //
 // Algorithmic flops: 4 * D per visible (query, key) pair and q head (QK^T + PV).
-#include <atomic>
 #include <type_traits>
 
 #include "msgl_device.h"
@@ -666,9 +665,10 @@ int launch_prefill_merge(const PrefillParams& p, int head_dim, hipStream_t strea
   return check_launch();
 }
 
-static std::atomic<int> g_tile_variant{0};
-int tile_variant() { return g_tile_variant.load(); }
-void set_tile_variant(int v) { g_tile_variant.store(v); }
+// benchmarking switch, one value per host thread (see msgl_set_tuning)
+static thread_local int t_tile_variant = 0;
+int tile_variant() { return t_tile_variant; }
+void set_tile_variant(int v) { t_tile_variant = v; }
 
 int launch_prefill_tile(const PrefillArgs& a, hipStream_t stream) {
   if (a.head_dim != 128) return MSGL_ERR_HEAD_DIM;

@@ -522,9 +522,9 @@ __global__ __launch_bounds__(64) void splitkv_merge_kernel(SplitKvParams p) {
 
 int nct_for(int64_t cols) { return (int)((cols + 15) / 16); }
 
-std::atomic<int> g_max_waves{4};
+thread_local int t_max_waves = 4;  // benchmarking switch, one value per host thread
 int heads_per_group(int64_t n_kv) {
-  const int cap = g_max_waves.load();
+  const int cap = t_max_waves;
   if (cap >= 8 && n_kv % 8 == 0) return 8;
   if (cap >= 4 && n_kv % 4 == 0) return 4;
   return (cap >= 2 && n_kv % 2 == 0) ? 2 : 1;
@@ -600,7 +600,7 @@ int launch_d(const SplitKvParams& p, int nct, hipStream_t stream) {
 
 }  // namespace
 
-void splitkv_set_max_waves(int v) { g_max_waves.store(v > 0 ? v : 4); }  // 0 restores the default
+void splitkv_set_max_waves(int v) { t_max_waves = v > 0 ? v : 4; }  // 0 restores the default
 
 // kv heads per workgroup for this shape: up to 4, halved when a second wave per head is
 // needed for the columns (a workgroup of the wide variants holds at most 4 waves: they

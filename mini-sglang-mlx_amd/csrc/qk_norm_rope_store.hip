@@ -36,7 +36,7 @@ struct NormRopeParams {
   uint16_t* q_out;
   uint16_t* k_cache;
   uint16_t* v_cache;
-  int64_t q_stride0, k_stride0, v_stride0, kc_stride0, vc_stride0;
+  int64_t q_stride0, k_stride0, v_stride0, kc_stride0, vc_stride0, num_slots;
   int32_t n_tokens, n_q, n_kv, chunks;  // chunks of kHeadsPerGroup heads per token
   float eps, log2_base;
 };
@@ -78,6 +78,9 @@ __global__ __launch_bounds__(kThreads) void qk_norm_rope_store_kernel(NormRopePa
     }
   }
   const int64_t slot = p.out_loc[t];
+  // a slot id outside the pools stores no k / v row (q_out is still produced): a wild store
+  // would be a GPU memory fault
+  const bool slot_ok = (uint64_t)slot < (uint64_t)p.num_slots;
   const int off = j * E;
 
   for (int h = h_begin; h < h_end; ++h) {
@@ -132,6 +135,7 @@ __global__ __launch_bounds__(kThreads) void qk_norm_rope_store_kernel(NormRopePa
         hi[e >> 1] = (uint32_t)oh[e] | ((uint32_t)oh[e + 1] << 16);
       }
     }
+    if (h >= p.n_q && !slot_ok) continue;
     *reinterpret_cast<V*>(dst + off) = lo;
     *reinterpret_cast<V*>(dst + D / 2 + off) = hi;
   }
@@ -156,6 +160,7 @@ int launch_qk_norm_rope_store(const NormRopeArgs& a, hipStream_t stream) {
   p.v_stride0 = a.v_stride0;
   p.kc_stride0 = a.kc_stride0;
   p.vc_stride0 = a.vc_stride0;
+  p.num_slots = a.num_slots;
   p.n_tokens = (int32_t)a.n_tokens;
   p.n_q = (int32_t)a.n_q;
   p.n_kv = (int32_t)a.n_kv;

@@ -14,6 +14,7 @@ store_kv_cache.cpp:22-63).
 """
 from __future__ import annotations
 
+import os
 from typing import Optional
 
 import torch
@@ -45,22 +46,31 @@ def _stream_ptr(stream, device) -> int:
 
 class _on_device:
     """``torch.cuda.device(dev)`` that costs nothing when ``dev`` is current already (the usual
-    case: one process per GPU)."""
+    case: one process per GPU), and, for a call with an explicit ``stream=``, that stream made
+    torch's current one for the duration of the call.  The second part is what makes a foreign
+    stream safe: the output, the workspace and any ``.contiguous()`` copy of an argument are
+    then allocated and produced on the stream the kernels run on, so torch's caching allocator
+    never hands one of these blocks to work that is still in flight on another stream."""
 
-    __slots__ = ("_guard",)
+    __slots__ = ("_guards",)
 
-    def __init__(self, dev: torch.device):
+    def __init__(self, dev: torch.device, stream=None):
+        self._guards = []
         index = dev.index
-        self._guard = None if index is None or index == torch.cuda.current_device() \
-            else torch.cuda.device(dev)
+        if index is not None and index != torch.cuda.current_device():
+            self._guards.append(torch.cuda.device(dev))
+        if stream is not None:
+            if not isinstance(stream, torch.cuda.Stream):
+                stream = torch.cuda.ExternalStream(int(stream.cuda_stream), device=dev)
+            self._guards.append(torch.cuda.stream(stream))
 
     def __enter__(self):
-        if self._guard is not None:
-            self._guard.__enter__()
+        for g in self._guards:
+            g.__enter__()
 
     def __exit__(self, *exc):
-        if self._guard is not None:
-            self._guard.__exit__(*exc)
+        for g in reversed(self._guards):
+            g.__exit__(*exc)
         return False
 
 
@@ -87,17 +97,66 @@ def _int32_1d(op: str, t: torch.Tensor, name: str) -> torch.Tensor:
     return t if t.is_contiguous() else t.contiguous()
 
 
+def _checks_on(validate: Optional[bool]) -> bool:
+    """Index validation is opt-in: ``validate=True`` on the call, or ``MSGL_DEBUG_CHECKS=1`` in
+    the environment for every call that does not say ``validate=False``.  It costs a few small
+    device reductions and ONE host synchronisation per call, so it is off by default, and it is
+    skipped while the current stream is being captured into a graph (a capture cannot sync)."""
+    if validate is None:
+        validate = os.environ.get("MSGL_DEBUG_CHECKS", "0") not in ("", "0")
+    if not validate:
+        return False
+    return not (torch.cuda.is_available() and torch.cuda.is_current_stream_capturing())
+
+
+def _validate_slot_ids(op: str, name: str, ids: torch.Tensor, num_slots: int,
+                       unique: bool = False) -> None:
+    """Every id inside ``[0, num_slots)`` and, for a store, no id twice.  The kernels read or
+    write ``pool[id]`` unchecked (a stray id is a wild access: a GPU memory fault, not a wrong
+    value; the writers skip such a row, the readers cannot), and two rows stored to one slot
+    race (store_kv_cache.metal:24-30 has the same hole; the reference's allocator hands out
+    distinct slots, scheduler/cache.py:45-57).  Works on any device: min, max and a sort there,
+    then one transfer of three numbers."""
+    if ids.numel() == 0:
+        return
+    lo, hi = torch.aminmax(ids)
+    dup = torch.zeros((), dtype=torch.int64, device=ids.device)
+    if unique and ids.numel() > 1:
+        srt = torch.sort(ids).values
+        dup = (srt[1:] == srt[:-1]).sum()
+    lo, hi, dup = (int(x) for x in torch.stack([lo.long(), hi.long(), dup]).tolist())
+    if lo < 0 or hi >= num_slots:
+        _fail(op, f"{name} holds slot ids outside [0, {num_slots}): min {lo}, max {hi}")
+    if dup:
+        _fail(op, f"{name} holds {dup} duplicate slot id(s); rows stored to one slot race")
+
+
+def _validate_indptr(op: str, name: str, indptr: torch.Tensor, limit: int, what: str) -> None:
+    """A CSR offset array must start at >= 0, never decrease and end inside the array it
+    indexes."""
+    first, last = indptr[0], indptr[-1]
+    down = (indptr[1:] < indptr[:-1]).sum() if indptr.numel() > 1 else torch.zeros_like(first)
+    first, last, down = (int(x) for x in torch.stack([first.long(), last.long(), down.long()]).tolist())
+    if first < 0 or down:
+        _fail(op, f"{name} must start at >= 0 and be non-decreasing")
+    if last > limit:
+        _fail(op, f"{name} ends at {last}, beyond the {limit} entries of {what}")
+
+
 def _check_rc(op: str, rc: int) -> None:
     if rc != 0:
         _fail(op, _lib.strerror(rc))
 
 
 def store_kv_cache(k_cache: torch.Tensor, v_cache: torch.Tensor, indices: torch.Tensor,
-                   k: torch.Tensor, v: torch.Tensor, *, stream=None) -> None:
+                   k: torch.Tensor, v: torch.Tensor, *, stream=None,
+                   validate: Optional[bool] = None) -> None:
     """In place: ``k_cache[indices[r]] = k[r]``, ``v_cache[indices[r]] = v[r]`` (bit copy).
 
     Drop-in for ``mini_sglang_mlx_kernel.store_kv_cache`` (store_kv_cache.cpp:14-107).
-    ``indices`` must be unique; duplicates race exactly as in the reference.
+    ``indices`` must be unique; duplicates race exactly as in the reference.  A slot id outside
+    the pool stores nothing.  ``validate=True`` (or ``MSGL_DEBUG_CHECKS=1``) checks range and
+    uniqueness first, at the price of one host synchronisation.
     """
     op = "store_kv_cache"
     if k_cache.dim() != 3 or v_cache.dim() != 3:
@@ -123,6 +182,8 @@ def store_kv_cache(k_cache: torch.Tensor, v_cache: torch.Tensor, indices: torch.
     dev = _require_device(op, k_cache, v_cache, indices, k, v)
     if length == 0:
         return
+    if _checks_on(validate):
+        _validate_slot_ids(op, "indices", indices, num_pages, unique=True)
     row = num_kv_heads * head_dim
 
     def _src(t):
@@ -130,10 +191,10 @@ def store_kv_cache(k_cache: torch.Tensor, v_cache: torch.Tensor, indices: torch.
             t = t.contiguous()
         return t, (t.stride(0) if t.shape[0] > 1 else row)
 
-    k, k_stride0 = _src(k)
-    v, v_stride0 = _src(v)
-    indices = indices if indices.is_contiguous() else indices.contiguous()
-    with _on_device(dev):
+    with _on_device(dev, stream):
+        k, k_stride0 = _src(k)
+        v, v_stride0 = _src(v)
+        indices = indices if indices.is_contiguous() else indices.contiguous()
         rc = _lib.load().msgl_store_kv_cache(
             k_cache.data_ptr(), v_cache.data_ptr(), indices.data_ptr(), k.data_ptr(),
             v.data_ptr(), length, num_kv_heads, head_dim, num_pages,
@@ -155,25 +216,24 @@ def _attention_dtype(op: str, q: torch.Tensor, k_cache: torch.Tensor, v_cache: t
     return _DTYPE_CODE[q.dtype]
 
 
-def _workspace(nbytes: int, dev, stream) -> Optional[torch.Tensor]:
-    """Scratch from torch's caching allocator; safe to drop right after the launch because
-    the allocator reuses a block only in stream order (``record_stream`` for a foreign one)."""
+def _workspace(nbytes: int, dev) -> Optional[torch.Tensor]:
+    """Scratch from torch's caching allocator, taken on the launch stream (see ``_on_device``):
+    safe to drop right after the launch because the allocator reuses a block in stream order."""
     if nbytes == 0:
         return None
-    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
-    if stream is not None:
-        ws.record_stream(stream)
-    return ws
+    return torch.empty(nbytes, dtype=torch.uint8, device=dev)
 
 
 def paged_decode_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                            kv_indptr: torch.Tensor, kv_indices: torch.Tensor,
                            num_kv_splits: torch.Tensor, sm_scale: float, max_kv_splits: int,
-                           *, stream=None) -> torch.Tensor:
+                           *, stream=None, validate: Optional[bool] = None) -> torch.Tensor:
     """GQA paged decode: ``q (batch, n_q, d)`` against the tokens listed in ``kv_indices``.
 
     Drop-in for ``mini_sglang_mlx_kernel.paged_decode_attention``
     (paged_decode_attention.cpp:15-73).  Returns ``(batch, n_q, d)`` in the dtype of ``q``.
+    ``validate=True`` (or ``MSGL_DEBUG_CHECKS=1``) first checks ``kv_indptr`` and that every
+    entry of ``kv_indices`` names a slot of the pool (one host synchronisation).
     """
     op = "paged_decode_attention"
     if q.dim() != 3:
@@ -203,16 +263,19 @@ def paged_decode_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torc
     if num_kv_splits.shape[0] != batch:
         _fail(op, "num_kv_splits must have batch entries")
     dev = _require_device(op, q, k_cache, v_cache, kv_indptr, kv_indices, num_kv_splits)
-    q = q if q.is_contiguous() else q.contiguous()
-    out = torch.empty((batch, num_q_heads, head_dim), dtype=q.dtype, device=dev)
-    if batch == 0:
-        return out
     lib = _lib.load()
     total_kv = kv_indices.shape[0]
-    with _on_device(dev):
+    if batch > 0 and _checks_on(validate):
+        _validate_indptr(op, "kv_indptr", kv_indptr, total_kv, "kv_indices")
+        _validate_slot_ids(op, "kv_indices", kv_indices, k_cache.shape[0])
+    with _on_device(dev, stream):
+        q = q if q.is_contiguous() else q.contiguous()
+        out = torch.empty((batch, num_q_heads, head_dim), dtype=q.dtype, device=dev)
+        if batch == 0:
+            return out
         ws_bytes = lib.msgl_paged_decode_workspace_bytes(batch, total_kv, num_q_heads,
                                                          num_kv_heads, head_dim)
-        ws = _workspace(ws_bytes, dev, stream)
+        ws = _workspace(ws_bytes, dev)
         rc = lib.msgl_paged_decode_attention(
             q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), kv_indptr.data_ptr(),
             kv_indices.data_ptr(), num_kv_splits.data_ptr(), out.data_ptr(),
@@ -229,7 +292,7 @@ def paged_prefill_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
                             kv_indices: torch.Tensor, prefix_lens: torch.Tensor,
                             sm_scale: float, max_len_extend: int, *,
                             is_cross_attention: bool = False, sliding_window_size: int = 0,
-                            stream=None) -> torch.Tensor:
+                            stream=None, validate: Optional[bool] = None) -> torch.Tensor:
     """Paged extend attention on top of a cached prefix.
 
     Drop-in for ``mini_sglang_mlx_kernel.paged_prefill_attention``
@@ -237,7 +300,9 @@ def paged_prefill_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
     ``prefix_lens[b] + i``; key ``j`` of the request is visible iff
     ``(is_cross_attention or j <= pos) and (W == 0 or j >= pos - W + 1)``.
     Returns ``(total_q, n_q, d)`` in the dtype of ``q``; rows of a request beyond
-    ``max_len_extend`` are not computed.
+    ``max_len_extend`` are not computed.  ``validate=True`` (or ``MSGL_DEBUG_CHECKS=1``) first
+    checks both offset arrays and that every entry of ``kv_indices`` names a slot of the pool
+    (one host synchronisation).
     """
     op = "paged_prefill_attention"
     if q.dim() != 3:
@@ -270,16 +335,20 @@ def paged_prefill_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
     if kv_indptr.shape[0] != batch + 1 or prefix_lens.shape[0] != batch:
         _fail(op, "kv_indptr / prefix_lens length must match qo_indptr")
     dev = _require_device(op, q, k_cache, v_cache, qo_indptr, kv_indptr, kv_indices, prefix_lens)
-    q = q if q.is_contiguous() else q.contiguous()
-    out = torch.empty((total_q, num_q_heads, head_dim), dtype=q.dtype, device=dev)
-    if total_q == 0:
-        return out
     lib = _lib.load()
     total_kv = kv_indices.shape[0]
-    with _on_device(dev):
+    if total_q > 0 and _checks_on(validate):
+        _validate_indptr(op, "qo_indptr", qo_indptr, total_q, "q")
+        _validate_indptr(op, "kv_indptr", kv_indptr, total_kv, "kv_indices")
+        _validate_slot_ids(op, "kv_indices", kv_indices, k_cache.shape[0])
+    with _on_device(dev, stream):
+        q = q if q.is_contiguous() else q.contiguous()
+        out = torch.empty((total_q, num_q_heads, head_dim), dtype=q.dtype, device=dev)
+        if total_q == 0:
+            return out
         ws_bytes = lib.msgl_paged_prefill_workspace_bytes(
             batch, total_q, total_kv, num_q_heads, num_kv_heads, head_dim, int(max_len_extend))
-        ws = _workspace(ws_bytes, dev, stream)
+        ws = _workspace(ws_bytes, dev)
         rc = lib.msgl_paged_prefill_attention(
             q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), qo_indptr.data_ptr(),
             kv_indptr.data_ptr(), kv_indices.data_ptr(), prefix_lens.data_ptr(), out.data_ptr(),
@@ -335,19 +404,20 @@ def build_attention_metadata(page_table: torch.Tensor, table_rows: torch.Tensor,
     # one allocation, six views (an allocation per array costs more host time than the kernel)
     sizes = (("kv_indptr", batch + 1), ("qo_indptr", batch + 1), ("prefix_lens", batch),
              ("num_kv_splits", batch), ("positions", total_q), ("kv_indices", total_kv))
-    buf = torch.empty(sum(n for _, n in sizes), dtype=torch.int32, device=dev)
-    out, at = {}, 0
-    for name, n in sizes:
-        out[name] = buf[at:at + n]
-        at += n
     rows = page_table.shape[0]
     stride0 = page_table.stride(0) if rows > 1 else page_table.shape[1]
-    rc = _lib.load().msgl_build_attention_metadata(
-        page_table.data_ptr(), stride0, rows, page_table.shape[1], table_rows.data_ptr(),
-        kv_lens.data_ptr(), extend_lens.data_ptr() if extend_lens is not None else None, batch,
-        out["kv_indptr"].data_ptr(), out["kv_indices"].data_ptr(), total_kv,
-        out["qo_indptr"].data_ptr(), out["prefix_lens"].data_ptr(), out["positions"].data_ptr(),
-        total_q, out["num_kv_splits"].data_ptr(), int(max_kv_splits), _stream_ptr(stream, dev))
+    with _on_device(dev, stream):
+        buf = torch.empty(sum(n for _, n in sizes), dtype=torch.int32, device=dev)
+        out, at = {}, 0
+        for name, n in sizes:
+            out[name] = buf[at:at + n]
+            at += n
+        rc = _lib.load().msgl_build_attention_metadata(
+            page_table.data_ptr(), stride0, rows, page_table.shape[1], table_rows.data_ptr(),
+            kv_lens.data_ptr(), extend_lens.data_ptr() if extend_lens is not None else None, batch,
+            out["kv_indptr"].data_ptr(), out["kv_indices"].data_ptr(), total_kv,
+            out["qo_indptr"].data_ptr(), out["prefix_lens"].data_ptr(), out["positions"].data_ptr(),
+            total_q, out["num_kv_splits"].data_ptr(), int(max_kv_splits), _stream_ptr(stream, dev))
     _check_rc(op, rc)
     return out
 
@@ -363,7 +433,8 @@ def _heads_stride0(op: str, t: torch.Tensor, name: str) -> int:
 def qk_norm_rope_store(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, q_weight: torch.Tensor,
                        k_weight: torch.Tensor, positions: torch.Tensor, out_loc: torch.Tensor,
                        k_cache: torch.Tensor, v_cache: torch.Tensor, *, eps: float,
-                       rope_base: float, stream=None) -> torch.Tensor:
+                       rope_base: float, stream=None,
+                       validate: Optional[bool] = None) -> torch.Tensor:
     """Per-head RMSNorm of q and k, rotary embedding of both at ``positions``, and the store of
     the new k and v rows at ``out_loc``, in one pass; returns the rotated q.
 
@@ -393,14 +464,18 @@ def qk_norm_rope_store(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, q_weig
     out_loc = _int32_1d(op, out_loc, "out_loc")
     if positions.shape[0] != n_tokens or out_loc.shape[0] != n_tokens:
         _fail(op, "positions and out_loc length must match q length")
-    q_out = torch.empty((n_tokens, n_q, d), dtype=q.dtype, device=dev)
-    rc = _lib.load().msgl_qk_norm_rope_store(
-        q.data_ptr(), k.data_ptr(), v.data_ptr(), qs, ks, vs, q_weight.contiguous().data_ptr(),
-        k_weight.contiguous().data_ptr(), positions.data_ptr(), out_loc.data_ptr(),
-        q_out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
-        _pool_stride0(op, k_cache, "k_cache"), _pool_stride0(op, v_cache, "v_cache"),
-        k_cache.shape[0], n_tokens, n_q, n_kv, d, float(eps), float(rope_base),
-        _lib.MSGL_DTYPE_BF16, _stream_ptr(stream, dev))
+    if _checks_on(validate):
+        _validate_slot_ids(op, "out_loc", out_loc, k_cache.shape[0], unique=True)
+    with _on_device(dev, stream):
+        q_out = torch.empty((n_tokens, n_q, d), dtype=q.dtype, device=dev)
+        q_weight, k_weight = q_weight.contiguous(), k_weight.contiguous()
+        rc = _lib.load().msgl_qk_norm_rope_store(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), qs, ks, vs, q_weight.data_ptr(),
+            k_weight.data_ptr(), positions.data_ptr(), out_loc.data_ptr(),
+            q_out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+            _pool_stride0(op, k_cache, "k_cache"), _pool_stride0(op, v_cache, "v_cache"),
+            k_cache.shape[0], n_tokens, n_q, n_kv, d, float(eps), float(rope_base),
+            _lib.MSGL_DTYPE_BF16, _stream_ptr(stream, dev))
     _check_rc(op, rc)
     return q_out
 
@@ -461,14 +536,16 @@ def gdn_state_inplace(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torc
     if not (state.stride(3) == 1 and state.stride(2) == dk and state.stride(1) == dv * dk):
         _fail(op, "state must be contiguous in its (hv, dv, dk) dimensions")
     state_stride0 = state.stride(0) if state.shape[0] > 1 else hv * dv * dk
-    g, beta = g.contiguous(), beta.contiguous()
-    slot_ids = slot_ids.contiguous()
-    y = torch.empty((tokens, hv, dv), dtype=q.dtype, device=dev)
-    rc = _lib.load().msgl_gdn_state_inplace(
-        q.data_ptr(), k.data_ptr(), v.data_ptr(), g.data_ptr(), beta.data_ptr(), state.data_ptr(),
-        slot_ids.data_ptr(), None if single_token_mode else qo_indptr.contiguous().data_ptr(),
-        y.data_ptr(), tokens, batch, hk, hv, dk, dv, state.shape[0], state_stride0, qs, ks, vs,
-        1 if single_token_mode else 0, _stream_ptr(stream, dev))
+    with _on_device(dev, stream):
+        g, beta = g.contiguous(), beta.contiguous()
+        slot_ids = slot_ids.contiguous()
+        qo_indptr = None if single_token_mode else qo_indptr.contiguous()
+        y = torch.empty((tokens, hv, dv), dtype=q.dtype, device=dev)
+        rc = _lib.load().msgl_gdn_state_inplace(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), g.data_ptr(), beta.data_ptr(), state.data_ptr(),
+            slot_ids.data_ptr(), None if qo_indptr is None else qo_indptr.data_ptr(),
+            y.data_ptr(), tokens, batch, hk, hv, dk, dv, state.shape[0], state_stride0, qs, ks, vs,
+            1 if single_token_mode else 0, _stream_ptr(stream, dev))
     _check_rc(op, rc)
     return y
 

@@ -8,7 +8,7 @@ already free (:160-168), ``check_ownership`` (:107-135), ``copy`` / ``copy_batch
 ``buf[dst] = buf[src]`` with every source read before any write (:170-189).
 
 Pinned by the twelve scenarios of the reference's mini_sglang_mlx/tests/test_mamba_slots.py
-(expected values restated in tests/_mamba_util.py).  bfloat16 buffers are kept as uint16 bit
+(expected values held as data in tests/golden/mamba_slot_scenarios.json).  bfloat16 buffers are kept as uint16 bit
 patterns: nothing here does arithmetic on them.
 """
 from __future__ import annotations

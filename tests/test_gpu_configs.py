@@ -93,10 +93,8 @@ def test_cfg4_long_context_decode_split_and_sampled_oracle(gpu):
     for segments in (16, 509):
         print(f"cfg4 segments={segments}", flush=True)
         _lib.set_tuning(_lib.TUNE_SEGMENTS, segments)
-        try:
-            other, _ = run_gpu(wl, gpu)
-        finally:
-            _lib.set_tuning(_lib.TUNE_SEGMENTS, 0)
+        other, _ = run_gpu(wl, gpu)
+        _lib.set_tuning(_lib.TUNE_SEGMENTS, 0)
         assert_close_bf16(other, got.float(), f"cfg4 split invariance ({segments})",
                           max_tol=4e-3, mean_tol=2e-4)
     reqs = _shortest(wl, 2)

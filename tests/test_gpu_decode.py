@@ -34,11 +34,9 @@ def test_decode_result_independent_of_the_split(gpu, segments, min_seg):
                         kv_lens=[5, 100, 257, 1000, 2049, 31, 64, 0, 640], pool_factor=1.2)
     _lib.set_tuning(_lib.TUNE_SEGMENTS, segments)
     _lib.set_tuning(_lib.TUNE_MIN_SEGMENT, min_seg)
-    try:
-        _check(wl, gpu, f"decode segments={segments} min_seg={min_seg}")
-    finally:
-        _lib.set_tuning(_lib.TUNE_SEGMENTS, 0)
-        _lib.set_tuning(_lib.TUNE_MIN_SEGMENT, 0)
+    _check(wl, gpu, f"decode segments={segments} min_seg={min_seg}")
+    _lib.set_tuning(_lib.TUNE_SEGMENTS, 0)
+    _lib.set_tuning(_lib.TUNE_MIN_SEGMENT, 0)
 
 
 def test_decode_empty_request_gives_zeros_and_page_size_one(gpu):
@@ -136,13 +134,11 @@ def test_decode_in_ieee_half_full_mantissa_inputs_and_split_invariance(gpu):
     outs = []
     for segments in (0, 1, 13):
         _lib.set_tuning(_lib.TUNE_SEGMENTS, segments)
-        try:
-            print(f"decode float16 dense, segments={segments}", flush=True)
-            out = paged_decode_attention(q.to(gpu), kc.to(gpu), vc.to(gpu), kv_indptr.to(gpu),
-                                         kv_indices.to(gpu), splits.to(gpu), d ** -0.5, 32)
-            torch.cuda.synchronize()
-        finally:
-            _lib.set_tuning(_lib.TUNE_SEGMENTS, 0)
+        print(f"decode float16 dense, segments={segments}", flush=True)
+        out = paged_decode_attention(q.to(gpu), kc.to(gpu), vc.to(gpu), kv_indptr.to(gpu),
+                                     kv_indices.to(gpu), splits.to(gpu), d ** -0.5, 32)
+        torch.cuda.synchronize()
+        _lib.set_tuning(_lib.TUNE_SEGMENTS, 0)
         assert_close_bf16(out, want, f"decode float16 dense segments={segments}",
                           max_tol=5e-3, mean_tol=4e-4)
         outs.append(out.float().cpu())

@@ -31,11 +31,9 @@ def test_tile_kernels_repeat_bit_identical(gpu, head_dim, splits, n_q, n_kv):
     g = wl.to(gpu)
     print(f"repeat tile head_dim={head_dim} splits={splits} heads={n_q}/{n_kv}", flush=True)
     _lib.set_tuning(_lib.TUNE_PREFILL_KEY_SPLITS, splits)
-    try:
-        outs = [_prefill(g, 257) for _ in range(RUNS)]
-        torch.cuda.synchronize()
-    finally:
-        _lib.set_tuning(_lib.TUNE_PREFILL_KEY_SPLITS, 0)
+    outs = [_prefill(g, 257) for _ in range(RUNS)]
+    torch.cuda.synchronize()
+    _lib.set_tuning(_lib.TUNE_PREFILL_KEY_SPLITS, 0)
     for i, out in enumerate(outs[1:], 1):
         assert torch.equal(out.view(torch.int16), outs[0].view(torch.int16)), f"run {i} differs from run 0"
 
@@ -127,12 +125,10 @@ def test_random_extend_shapes_repeat_bit_identical(gpu, seed):
     print(f"repeat random seed={seed} heads={n_q}/{n_kv} d={d} ext={ext} kv={kv} cross={is_cross} "
           f"W={window} key_splits={splits}", flush=True)
     _lib.set_tuning(_lib.TUNE_PREFILL_KEY_SPLITS, splits)
-    try:
-        outs = [_prefill(g, max(ext), is_cross_attention=is_cross, sliding_window_size=window)
-                for _ in range(12)]
-        torch.cuda.synchronize()
-    finally:
-        _lib.set_tuning(_lib.TUNE_PREFILL_KEY_SPLITS, 0)
+    outs = [_prefill(g, max(ext), is_cross_attention=is_cross, sliding_window_size=window)
+            for _ in range(12)]
+    torch.cuda.synchronize()
+    _lib.set_tuning(_lib.TUNE_PREFILL_KEY_SPLITS, 0)
     for i, out in enumerate(outs[1:], 1):
         assert torch.equal(out.view(torch.int16), outs[0].view(torch.int16)), f"run {i} differs from run 0"
 

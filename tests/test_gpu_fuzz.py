@@ -58,10 +58,8 @@ def test_random_prefill_shapes(gpu, seed):
     from mini_sglang_amd_kernel import _lib
 
     _lib.set_tuning(_lib.TUNE_PREFILL_KEY_SPLITS, splits)
-    try:
-        got, g = run_gpu(wl, gpu)
-    finally:
-        _lib.set_tuning(_lib.TUNE_PREFILL_KEY_SPLITS, 0)
+    got, g = run_gpu(wl, gpu)
+    _lib.set_tuning(_lib.TUNE_PREFILL_KEY_SPLITS, 0)
     want, ref = run_oracle(wl)
     assert_close_bf16(got, want, what)
     if wl.out_loc is not None:

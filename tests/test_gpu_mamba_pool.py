@@ -4,7 +4,7 @@ import numpy as np
 import pytest
 import torch
 
-from _mamba_util import CONV_SHAPE, SCENARIOS, TEMPORAL_SHAPE
+from _slot_scenarios import CONV_SHAPE, SCENARIO_NAMES, TEMPORAL_SHAPE, run_scenario
 from mini_sglang_amd.kvcache import (MambaStateConfig, MambaStatePool,
                                      create_hybrid_radix_cache_manager)
 from oracle.mamba_pool_oracle import MambaPoolOracle
@@ -41,11 +41,11 @@ class GpuHarness:
                         device=cls.device)
 
 
-@pytest.mark.parametrize("scenario", SCENARIOS, ids=lambda f: f.__name__)
+@pytest.mark.parametrize("scenario", SCENARIO_NAMES)
 def test_reference_scenarios(gpu, scenario):
     GpuHarness.device = gpu
-    print(scenario.__name__, flush=True)
-    scenario(GpuHarness)
+    print(scenario, flush=True)
+    run_scenario(scenario, GpuHarness)
 
 
 def _random_pools(gpu, num_slots, layers, conv_shapes, temporal_shapes, seed):

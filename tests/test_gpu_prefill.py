@@ -254,11 +254,9 @@ def test_splitk_route_ragged_q_and_chunking(gpu):
     for segments in (1, 5, 64, 0):
         _lib.set_tuning(_lib.TUNE_SEGMENTS, segments)
         _lib.set_tuning(_lib.TUNE_MIN_SEGMENT, 64)
-        try:
-            _check(wl, gpu, f"split-K route ragged segments={segments}")
-        finally:
-            _lib.set_tuning(_lib.TUNE_SEGMENTS, 0)
-            _lib.set_tuning(_lib.TUNE_MIN_SEGMENT, 0)
+        _check(wl, gpu, f"split-K route ragged segments={segments}")
+        _lib.set_tuning(_lib.TUNE_SEGMENTS, 0)
+        _lib.set_tuning(_lib.TUNE_MIN_SEGMENT, 0)
 
 
 def test_both_routes_agree_and_decode_equals_prefill_qlen1(gpu):
@@ -268,10 +266,8 @@ def test_both_routes_agree_and_decode_equals_prefill_qlen1(gpu):
                         extend_lens=[8, 8, 8], pool_factor=1.0)
     a, _ = run_gpu(wl, gpu)
     _lib.set_tuning(_lib.TUNE_SMALLQ_MAXCOLS, -1)  # force the tile kernel
-    try:
-        b, _ = run_gpu(wl, gpu)
-    finally:
-        _lib.set_tuning(_lib.TUNE_SMALLQ_MAXCOLS, 0)
+    b, _ = run_gpu(wl, gpu)
+    _lib.set_tuning(_lib.TUNE_SMALLQ_MAXCOLS, 0)
     want, _ = run_oracle(wl)
     assert_close_bf16(a, want, "split-K route")
     assert_close_bf16(b, want, "tile route")
@@ -364,36 +360,34 @@ def test_key_split_equals_one_pass_and_leaves_capped_rows_alone(gpu, head_dim):
     for k in (1, 5):
         print(f"key splits {k} head_dim {head_dim} cap {cap}", flush=True)
         _lib.set_tuning(_lib.TUNE_PREFILL_KEY_SPLITS, k)
-        try:
-            out = torch.full_like(g.q, 7.0)
-            total_q, n_q, d = g.q.shape
-            batch, total_kv = g.qo_indptr.shape[0] - 1, g.kv_indices.shape[0]
-            ws_bytes = lib.msgl_paged_prefill_workspace_bytes(batch, total_q, total_kv, n_q,
-                                                              g.k_cache.shape[1], d, cap)
-            assert (ws_bytes > 0) == (k > 1)
-            ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=gpu)
-            rc = lib.msgl_paged_prefill_attention(
+        out = torch.full_like(g.q, 7.0)
+        total_q, n_q, d = g.q.shape
+        batch, total_kv = g.qo_indptr.shape[0] - 1, g.kv_indices.shape[0]
+        ws_bytes = lib.msgl_paged_prefill_workspace_bytes(batch, total_q, total_kv, n_q,
+                                                          g.k_cache.shape[1], d, cap)
+        assert (ws_bytes > 0) == (k > 1)
+        ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=gpu)
+        rc = lib.msgl_paged_prefill_attention(
+            g.q.data_ptr(), g.k_cache.data_ptr(), g.v_cache.data_ptr(), g.qo_indptr.data_ptr(),
+            g.kv_indptr.data_ptr(), g.kv_indices.data_ptr(), g.prefix_lens.data_ptr(),
+            out.data_ptr(), ws.data_ptr(), ws_bytes, batch, total_q, total_kv, n_q,
+            g.k_cache.shape[1], d, g.k_cache.shape[0], g.k_cache.stride(0), g.v_cache.stride(0),
+            float(g.sm_scale), cap, 0, 0, 0, None)
+        assert rc == 0, _lib.strerror(rc)
+        torch.cuda.synchronize()
+        if k > 1:  # too small a workspace is not overrun: the keys go in one pass
+            again = torch.full_like(g.q, 7.0)
+            ws.fill_(0x7f)
+            assert lib.msgl_paged_prefill_attention(
                 g.q.data_ptr(), g.k_cache.data_ptr(), g.v_cache.data_ptr(), g.qo_indptr.data_ptr(),
                 g.kv_indptr.data_ptr(), g.kv_indices.data_ptr(), g.prefix_lens.data_ptr(),
-                out.data_ptr(), ws.data_ptr(), ws_bytes, batch, total_q, total_kv, n_q,
-                g.k_cache.shape[1], d, g.k_cache.shape[0], g.k_cache.stride(0), g.v_cache.stride(0),
-                float(g.sm_scale), cap, 0, 0, 0, None)
-            assert rc == 0, _lib.strerror(rc)
+                again.data_ptr(), ws.data_ptr(), ws_bytes - 1, batch, total_q, total_kv, n_q,
+                g.k_cache.shape[1], d, g.k_cache.shape[0], g.k_cache.stride(0),
+                g.v_cache.stride(0), float(g.sm_scale), cap, 0, 0, 0, None) == 0
             torch.cuda.synchronize()
-            if k > 1:  # too small a workspace is not overrun: the keys go in one pass
-                again = torch.full_like(g.q, 7.0)
-                ws.fill_(0x7f)
-                assert lib.msgl_paged_prefill_attention(
-                    g.q.data_ptr(), g.k_cache.data_ptr(), g.v_cache.data_ptr(), g.qo_indptr.data_ptr(),
-                    g.kv_indptr.data_ptr(), g.kv_indices.data_ptr(), g.prefix_lens.data_ptr(),
-                    again.data_ptr(), ws.data_ptr(), ws_bytes - 1, batch, total_q, total_kv, n_q,
-                    g.k_cache.shape[1], d, g.k_cache.shape[0], g.k_cache.stride(0),
-                    g.v_cache.stride(0), float(g.sm_scale), cap, 0, 0, 0, None) == 0
-                torch.cuda.synchronize()
-                assert torch.equal(again.cpu().view(torch.int16), outs[0].view(torch.int16))
-                assert (ws == 0x7f).all()
-        finally:
-            _lib.set_tuning(_lib.TUNE_PREFILL_KEY_SPLITS, 0)
+            assert torch.equal(again.cpu().view(torch.int16), outs[0].view(torch.int16))
+            assert (ws == 0x7f).all()
+        _lib.set_tuning(_lib.TUNE_PREFILL_KEY_SPLITS, 0)
         outs.append(out.cpu())
     tail = slice(90 + cap, 90 + 120)
     for out in outs:
@@ -435,7 +429,5 @@ def test_partially_filled_query_blocks_idle_waves(gpu, head_dim):
                         kv_lens=[700 + 37 * i + e for i, e in enumerate(ext)], extend_lens=ext,
                         pool_factor=1.2, store_new=True)
     _lib.set_tuning(_lib.TUNE_SMALLQ_MAXCOLS, -1)
-    try:
-        _check(wl, gpu, f"partially filled query blocks head_dim={head_dim}")
-    finally:
-        _lib.set_tuning(_lib.TUNE_SMALLQ_MAXCOLS, 0)
+    _check(wl, gpu, f"partially filled query blocks head_dim={head_dim}")
+    _lib.set_tuning(_lib.TUNE_SMALLQ_MAXCOLS, 0)

@@ -34,9 +34,6 @@ def test_library_loads_and_exports_every_declared_symbol():
     assert _lib.strerror(0) == "ok"
     assert "head_dim" in _lib.strerror(-2)
     assert _lib.strerror(-9999) == "unknown error code"
-    # the benchmarking aid bench.py loads next to it
-    probes = ctypes.CDLL(os.path.join(os.path.dirname(_lib.LIB_PATH), "libmsgl_probes.so"))
-    assert hasattr(probes, "msgl_probe_mfma_rate")
 
 
 def test_c_abi_argument_checks_return_codes_without_touching_a_gpu():
@@ -275,3 +272,45 @@ def test_workload_generators_are_consistent():
     assert roofline.visible_pairs(prefix=6, q_len=2, kv_len=8, is_cross=True, window=3) == 4 + 3
     assert roofline.visible_range(6, 2, 8, True, 3) == (4, 8)
     assert roofline.decode_bytes([10], 4, 2, 128) == 10 * (2 * 2 * 128 * 2 + 4) + 2 * 4 * 128 * 2
+
+
+# ---- opt-in index validation in front of the launches (host-forcible: plain tensors) -----------
+def test_slot_id_validation_names_range_and_duplicates():
+    import mini_sglang_amd_kernel as mk
+
+    ok = torch.tensor([5, 0, 3], dtype=torch.int32)
+    mk._validate_slot_ids("store_kv_cache", "indices", ok, 6, unique=True)
+    mk._validate_slot_ids("store_kv_cache", "indices", ok[:0], 0, unique=True)  # nothing to check
+    for bad in ([1, 6], [-1, 2], [2 ** 31 - 1]):
+        with pytest.raises(RuntimeError, match=r"store_kv_cache: indices holds slot ids outside \[0, 6\)"):
+            mk._validate_slot_ids("store_kv_cache", "indices", torch.tensor(bad, dtype=torch.int32), 6)
+    twice = torch.tensor([4, 2, 4, 2, 1], dtype=torch.int32)
+    with pytest.raises(RuntimeError, match="2 duplicate slot id"):
+        mk._validate_slot_ids("store_kv_cache", "indices", twice, 6, unique=True)
+    mk._validate_slot_ids("paged_decode_attention", "kv_indices", twice, 6)  # readers may repeat
+
+
+def test_indptr_validation():
+    import mini_sglang_amd_kernel as mk
+
+    t = lambda v: torch.tensor(v, dtype=torch.int32)
+    mk._validate_indptr("op", "kv_indptr", t([0, 4, 4, 9]), 9, "kv_indices")
+    with pytest.raises(RuntimeError, match="non-decreasing"):
+        mk._validate_indptr("op", "kv_indptr", t([0, 4, 3]), 9, "kv_indices")
+    with pytest.raises(RuntimeError, match="non-decreasing"):
+        mk._validate_indptr("op", "kv_indptr", t([-1, 4]), 9, "kv_indices")
+    with pytest.raises(RuntimeError, match="ends at 10, beyond the 9 entries of kv_indices"):
+        mk._validate_indptr("op", "kv_indptr", t([0, 10]), 9, "kv_indices")
+
+
+def test_validation_is_off_unless_asked_for(monkeypatch):
+    import mini_sglang_amd_kernel as mk
+
+    monkeypatch.delenv("MSGL_DEBUG_CHECKS", raising=False)
+    assert mk._checks_on(None) is False and mk._checks_on(False) is False
+    assert mk._checks_on(True) is True
+    monkeypatch.setenv("MSGL_DEBUG_CHECKS", "1")
+    assert mk._checks_on(None) is True
+    assert mk._checks_on(False) is False  # the call's own word wins
+    monkeypatch.setenv("MSGL_DEBUG_CHECKS", "0")
+    assert mk._checks_on(None) is False

@@ -2,7 +2,7 @@
 import numpy as np
 import pytest
 
-from _mamba_util import CONV_SHAPE, SCENARIOS, TEMPORAL_SHAPE
+from _slot_scenarios import CONV_SHAPE, SCENARIO_NAMES, TEMPORAL_SHAPE, run_scenario
 from oracle.mamba_pool_oracle import MambaPoolOracle
 
 _BF16 = {0.0: 0x0000, 3.0: 0x4040, 5.0: 0x40A0, 7.0: 0x40E0}  # bit patterns of the values used
@@ -39,9 +39,9 @@ class OracleHarness:
                            [TEMPORAL_SHAPE] * num_layers, verify_width)
 
 
-@pytest.mark.parametrize("scenario", SCENARIOS, ids=lambda f: f.__name__)
+@pytest.mark.parametrize("scenario", SCENARIO_NAMES)
 def test_reference_scenarios(scenario):
-    scenario(OracleHarness)
+    run_scenario(scenario, OracleHarness)
 
 
 def test_copy_batched_reads_every_source_before_it_writes():
