@@ -59,6 +59,7 @@ extern "C" {
 #define MSGL_ERR_LAUNCH (-11)           /* the HIP runtime refused a launch (hipGetLastError) */
 #define MSGL_ERR_HEAD_DIM_MULT4 (-12)   /* store: head_dim is not a multiple of 4 */
 #define MSGL_ERR_GDN_DIMS (-13)         /* gdn_state_inplace: dk and dv must both be 128 */
+#define MSGL_ERR_SCRATCH_LIMIT (-14)    /* *_noalloc: sizes exceed the built-in scratch */
 
 /* Library version: major*10000 + minor*100 + patch. */
 MSGL_API int msgl_version(void);
@@ -112,6 +113,33 @@ MSGL_API int msgl_paged_decode_attention(const void* q, const void* k_cache, con
                                 const int32_t* kv_indptr, const int32_t* kv_indices,
                                 const int32_t* num_kv_splits, void* out,
                                 void* workspace, size_t workspace_bytes,
+                                int64_t batch, int64_t total_kv,
+                                int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim,
+                                int64_t num_slots,
+                                int64_t k_cache_stride0, int64_t v_cache_stride0,
+                                float sm_scale, int32_t max_kv_splits,
+                                int32_t dtype, void* stream);
+
+/*
+ * paged_decode_attention for callers that cannot allocate -- no counterpart in the reference
+ * (its decode op allocates att_out / att_lse on every call, paged_decode_attention.cpp:118-129).
+ * For code under HIP graph capture, tight serving loops and harnesses that forbid hipMalloc:
+ * same arguments and same result (bit for bit) as msgl_paged_decode_attention, minus the
+ * workspace, which is a file-scope device array of MSGL_DECODE_SCRATCH_BYTES that is part of
+ * the library's code object (every GPU the library runs on holds it until the process ends).
+ * The call makes no hipMalloc / hipFree and no allocating library call; the first call on a
+ * device looks the array's address up (hipGetSymbolAddress) and keeps it, so make that first
+ * call outside a capture.  Sizes whose split-K partials need more than the array
+ * ((segments + batch) * num_q_heads * (head_dim + 1) floats; 3.2 MB at batch 64, 32 / 8 heads
+ * of 128) return MSGL_ERR_SCRATCH_LIMIT and launch nothing.  Every call on one GPU uses the
+ * same array, whatever the stream: calls that overlap in time on one GPU race.  Nothing in the
+ * array has to start at zero (the attention kernel writes every entry the merge reads).
+ */
+#define MSGL_DECODE_SCRATCH_BYTES (8 * 1024 * 1024)
+MSGL_API int msgl_paged_decode_attention_noalloc(const void* q, const void* k_cache,
+                                const void* v_cache,
+                                const int32_t* kv_indptr, const int32_t* kv_indices,
+                                const int32_t* num_kv_splits, void* out,
                                 int64_t batch, int64_t total_kv,
                                 int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim,
                                 int64_t num_slots,

@@ -74,6 +74,9 @@ const char* msgl_strerror(int code) {
     case MSGL_ERR_LAUNCH: return "HIP kernel launch failed";
     case MSGL_ERR_HEAD_DIM_MULT4: return "head_dim must be a multiple of 4";
     case MSGL_ERR_GDN_DIMS: return "this specialized kernel requires dk=dv=128";
+    case MSGL_ERR_SCRATCH_LIMIT:
+      return "sizes need more split-K scratch than the library's built-in 8 MiB; use the entry "
+             "point that takes a workspace";
     default: return "unknown error code";
   }
 }
@@ -128,14 +131,16 @@ size_t msgl_paged_decode_workspace_bytes(int64_t batch, int64_t total_kv, int64_
                                        segments(total_kv, num_kv_heads, head_dim, group));
 }
 
-int msgl_paged_decode_attention(const void* q, const void* k_cache, const void* v_cache,
-                                const int32_t* kv_indptr, const int32_t* kv_indices,
-                                const int32_t* num_kv_splits, void* out, void* workspace,
-                                size_t workspace_bytes, int64_t batch, int64_t total_kv,
-                                int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim,
-                                int64_t num_slots, int64_t k_cache_stride0,
-                                int64_t v_cache_stride0, float sm_scale, int32_t max_kv_splits,
-                                int32_t dtype, void* stream) {
+// Both decode entry points: `builtin_scratch` takes the workspace from the library's own
+// per-device array instead of the caller.
+static int decode_attention(const void* q, const void* k_cache, const void* v_cache,
+                            const int32_t* kv_indptr, const int32_t* kv_indices,
+                            const int32_t* num_kv_splits, void* out, void* workspace,
+                            size_t workspace_bytes, bool builtin_scratch, int64_t batch,
+                            int64_t total_kv, int64_t num_q_heads, int64_t num_kv_heads,
+                            int64_t head_dim, int64_t num_slots, int64_t k_cache_stride0,
+                            int64_t v_cache_stride0, float sm_scale, int32_t max_kv_splits,
+                            int32_t dtype, void* stream) {
   if (batch < 0 || total_kv < 0 || num_slots < 0) return MSGL_ERR_SHAPE;
   if (batch == 0) return MSGL_OK;
   int rc = check_common(q, k_cache, v_cache, out, num_q_heads, num_kv_heads, head_dim,
@@ -148,6 +153,11 @@ int msgl_paged_decode_attention(const void* q, const void* k_cache, const void* 
   const int32_t n_seg = segments(total_kv, num_kv_heads, head_dim, group);
   const size_t need =
       msgl::splitkv_workspace_bytes(batch, num_q_heads, num_kv_heads, head_dim, 1, n_seg);
+  if (builtin_scratch) {
+    rc = msgl::splitkv_scratch(&workspace, &workspace_bytes);
+    if (rc != MSGL_OK) return rc;
+    if (need > workspace_bytes) return MSGL_ERR_SCRATCH_LIMIT;
+  }
   if (!workspace || workspace_bytes < need || !aligned16(workspace)) return MSGL_ERR_WORKSPACE;
   msgl::SplitKvArgs a{};
   a.q = q;
@@ -175,6 +185,33 @@ int msgl_paged_decode_attention(const void* q, const void* k_cache, const void* 
   a.n_seg = n_seg;
   a.min_seg = min_segment();
   return msgl::launch_splitkv(a, static_cast<hipStream_t>(stream));
+}
+
+int msgl_paged_decode_attention(const void* q, const void* k_cache, const void* v_cache,
+                                const int32_t* kv_indptr, const int32_t* kv_indices,
+                                const int32_t* num_kv_splits, void* out, void* workspace,
+                                size_t workspace_bytes, int64_t batch, int64_t total_kv,
+                                int64_t num_q_heads, int64_t num_kv_heads, int64_t head_dim,
+                                int64_t num_slots, int64_t k_cache_stride0,
+                                int64_t v_cache_stride0, float sm_scale, int32_t max_kv_splits,
+                                int32_t dtype, void* stream) {
+  return decode_attention(q, k_cache, v_cache, kv_indptr, kv_indices, num_kv_splits, out, workspace,
+                          workspace_bytes, false, batch, total_kv, num_q_heads, num_kv_heads,
+                          head_dim, num_slots, k_cache_stride0, v_cache_stride0, sm_scale,
+                          max_kv_splits, dtype, stream);
+}
+
+int msgl_paged_decode_attention_noalloc(const void* q, const void* k_cache, const void* v_cache,
+                                        const int32_t* kv_indptr, const int32_t* kv_indices,
+                                        const int32_t* num_kv_splits, void* out, int64_t batch,
+                                        int64_t total_kv, int64_t num_q_heads,
+                                        int64_t num_kv_heads, int64_t head_dim, int64_t num_slots,
+                                        int64_t k_cache_stride0, int64_t v_cache_stride0,
+                                        float sm_scale, int32_t max_kv_splits, int32_t dtype,
+                                        void* stream) {
+  return decode_attention(q, k_cache, v_cache, kv_indptr, kv_indices, num_kv_splits, out, nullptr,
+                          0, true, batch, total_kv, num_q_heads, num_kv_heads, head_dim, num_slots,
+                          k_cache_stride0, v_cache_stride0, sm_scale, max_kv_splits, dtype, stream);
 }
 
 static bool use_splitkv_route(int64_t group, int64_t max_len_extend) {

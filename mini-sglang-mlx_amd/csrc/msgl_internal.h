@@ -49,6 +49,9 @@ int splitkv_default_segments(int64_t total_kv, int64_t n_kv, int64_t head_dim, i
 size_t splitkv_workspace_bytes(int64_t batch, int64_t n_q, int64_t n_kv, int64_t head_dim,
                                int64_t max_len_extend, int32_t n_seg);
 int launch_splitkv(const SplitKvArgs& a, hipStream_t stream);
+// Address (on the current device) and size of the library's built-in split-K scratch, for the
+// entry point that takes no workspace.  The first call on a device resolves the address.
+int splitkv_scratch(void** ptr, size_t* bytes);
 // benchmarking switch: most waves (adjacent kv heads) a split-K workgroup may hold
 void splitkv_set_max_waves(int v);
 

@@ -600,6 +600,34 @@ int launch_d(const SplitKvParams& p, int nct, hipStream_t stream) {
 
 }  // namespace
 
+// ---- built-in scratch for callers that cannot allocate --------------------------------------
+// One array per GPU, part of the loaded code object, held until the process ends.  In host code
+// the array's name is only a handle for hipGetSymbolAddress: the address that kernels and copies
+// use is looked up once per device, with that device current, and kept.
+constexpr size_t kScratchBytes = (size_t)MSGL_DECODE_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+int splitkv_scratch(void** ptr, size_t* bytes) {
+  constexpr int kMaxDevices = 64;
+  static std::atomic<void*> addr[kMaxDevices];
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    (void)hipGetLastError();
+    return MSGL_ERR_LAUNCH;
+  }
+  void* p = addr[dev].load(std::memory_order_acquire);
+  if (p == nullptr) {
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || p == nullptr) {
+      (void)hipGetLastError();
+      return MSGL_ERR_LAUNCH;
+    }
+    addr[dev].store(p, std::memory_order_release);  // every thread resolves the same address
+  }
+  *ptr = p;
+  *bytes = kScratchBytes;
+  return MSGL_OK;
+}
+
 void splitkv_set_max_waves(int v) { t_max_waves = v > 0 ? v : 4; }  // 0 restores the default
 
 // kv heads per workgroup for this shape: up to 4, halved when a second wave per head is

@@ -32,6 +32,10 @@ SIGNATURES = {
         ctypes.c_int,
         [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i64, _i64, _i64, _i64, _i64, _i64,
          _i64, _i64, _f32, _i32, _i32, _vp]),
+    "msgl_paged_decode_attention_noalloc": (
+        ctypes.c_int,
+        [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64,
+         _i64, _i64, _f32, _i32, _i32, _vp]),
     "msgl_paged_prefill_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64, _i64, _i64, _i64]),
     "msgl_paged_prefill_attention": (
         ctypes.c_int,
