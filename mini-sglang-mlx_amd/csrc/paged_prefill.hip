@@ -175,11 +175,12 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
     for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
       for (int i = 0; i < 16; ++i) oacc[dt][rt][i] = 0.f;
-  float m_run[RT], l_run[RT];
+  float m_run[RT], l_run[RT], m_safe_run[RT];  // m_safe_run: m_run, or 0 while m_run is -inf
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
     m_run[rt] = kNegInf;
     l_run[rt] = 0.f;
+    m_safe_run[rt] = 0.f;
   }
 
   // ---- moving a tile: wave w owns units w*UPW .. w*UPW+UPW-1; in a unit, lane l fetches
@@ -310,6 +311,22 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
     }
   };
   auto decide = [&](const float (&mx)[RT], Stats& st) {
+    // Usual case: no lane of the wave saw a score more than kLazy above its row's running max.
+    // Then no row's max moves (the other half of a row sits in this wave too), the state stays
+    // as it is, and the cross-lane exchange, the selects and the exponential below are skipped:
+    // one multiply, one compare and a scalar branch instead of a dozen instructions and an LDS
+    // round trip.  The first tile (running max -inf) and fully masked halves take the long way.
+    bool grew = false;
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) grew |= (mx[rt] * st.mul > m_run[rt] + kLazy);
+    if (!__any(grew)) {
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        st.m_safe[rt] = m_safe_run[rt];
+        st.alpha[rt] = 1.0f;
+      }
+      return;
+    }
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
       const float m = wave_max_xor(mx[rt] * st.mul, 32);
@@ -317,6 +334,7 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
       const float m_new = fmaxf(m_old, m);
       const float m_use = (m_new - m_old > kLazy) ? m_new : m_old;
       st.m_safe[rt] = (m_use == kNegInf) ? 0.f : m_use;
+      m_safe_run[rt] = st.m_safe[rt];
       st.alpha[rt] = fast_exp2(m_old - st.m_safe[rt]);
       m_run[rt] = m_use;
       pin(st.m_safe[rt]);
