@@ -624,6 +624,494 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
 }
 
 
+// =============================================================================================
+// Ping-pong variant of the tile kernel (same tiling, same LDS layout, same data path).
+//
+// The two waves that share a SIMD (w and w + 4) never do the same kind of work at the same
+// time.  Time is cut into slots separated by workgroup barriers; in every slot the waves of one
+// group (w < 4, one per SIMD) run an M phase, nothing but MFMAs and their LDS operand reads:
+//     O^T += V(j)^T P(j)^T,   S(j+1)^T = K(j+1) Q^T            (32 MFMAs, a whole 64-key tile)
+// while the waves of the other group run a V phase, nothing but VALU and the tile moves:
+//     P(j+1) = softmax step of S(j+1)  (row max, lazy rescale, exp2, bf16 pack, row sum)
+// and then they swap.  The matrix pipe of a SIMD therefore always has exactly one wave feeding
+// it, and that wave's softmax never competes with its own or its partner's MFMAs for issue
+// slots in the same phase of the instruction stream.
+//
+//   slot      0       1       2       3       4      ...
+//   w < 4   M(-1)   V(-1)   M(0)    V(0)    M(1)           M(-1): scores of tile 0 only
+//   w >= 4   -      M(-1)   V(-1)   M(0)    V(0)
+//
+// Tiles: K(t) and V(t) live in stage t % 4 of four K and four V stages.  M phase j, whose wave
+// has issue slots to spare between its MFMAs, also sends K(j+4) and V(j+3) on their way (each
+// wave its two units of each) and, at its end, waits for what it sent in M phase j-1, so a tile
+// is in flight for two slots and has been published by a barrier a full slot before its first
+// reader asks for operands.  The slot ids of a tile travel through a small LDS ring of the
+// wave's own (one dword LDS-direct load per tile, two M phases ahead; read back into registers
+// at the end of the M phase before the one that uses them), which keeps every vector-memory
+// operation of the loop out of the compiler's wait bookkeeping: the only vector-memory wait in
+// the loop is the counted one at the end of an M phase.  Order of issue inside an M phase:
+// [ring fetch, 4 moves].
+#ifndef MSGL_PP_PRIO_M
+#define MSGL_PP_PRIO_M 3
+#endif
+#ifndef MSGL_PP_PRIO_V
+#define MSGL_PP_PRIO_V 0
+#endif
+namespace pp {
+constexpr int kStages = 4;
+constexpr int kVBase = kStages * kKStage;
+constexpr int kRingBase = kVBase + kStages * kVStage;
+constexpr int kRingStage = 256;  // one dword per lane
+constexpr int kRingStages = 4;
+constexpr int kRingWave = kRingStages * kRingStage;
+constexpr int kSmem = kRingBase + 8 * kRingWave;
+}  // namespace pp
+
+template <bool WIDE>
+__global__ __launch_bounds__(512) void prefill_pingpong_kernel(PrefillParams p) {
+  constexpr int D = 128, NW = 8, UPW = kUnits / NW, KSTEPS = D / 16, DT = D / 32;
+  constexpr int kRows = NW * 32;
+  constexpr int OROW = D + 8;
+  static_assert(kRows * OROW * 2 <= pp::kSmem, "output staging must fit the stages");
+  __shared__ __attribute__((aligned(16))) unsigned char smem[pp::kSmem];
+  using OffT = typename std::conditional<WIDE, uint64_t, uint32_t>::type;
+
+  const int tid = threadIdx.x;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lane = tid & 63;
+  const int h = lane >> 5;
+  const int c32 = lane & 31;
+
+  // ---- block -> (request, kv head, key split, q block): as in prefill_tile_kernel ----------
+  const int xcd = blockIdx.x & 7;
+  const int seq = blockIdx.x >> 3;
+  const int unit = (seq / p.n_qblk) * 8 + xcd;
+  if (unit >= p.n_pairs * p.n_ksplit) return;
+  const int pair = unit / p.n_ksplit;
+  const int split = unit - pair * p.n_ksplit;
+  const int qblk = p.n_qblk - 1 - (seq % p.n_qblk);
+  const int want_rank = pair / p.n_kv;
+  const int kvh = pair - want_rank * p.n_kv;
+  __shared__ int ranked_request;
+  if (p.batch <= kRankedBatch) {
+    for (int i = tid; i < p.batch; i += NW * 64) {
+      const int len_i = p.kv_indptr[i + 1] - p.kv_indptr[i];
+      int rank = 0;
+      for (int j = 0; j < p.batch; ++j) {
+        const int len_j = p.kv_indptr[j + 1] - p.kv_indptr[j];
+        rank += (len_j > len_i) || (len_j == len_i && j < i);
+      }
+      if (rank == want_rank) ranked_request = i;
+    }
+  } else if (tid == 0) {
+    ranked_request = want_rank;
+  }
+  __syncthreads();
+  const int b = ranked_request;
+
+  const int q_start = p.qo_indptr[b];
+  const int q_len = min(p.qo_indptr[b + 1] - q_start, p.max_len_extend);
+  const int kv_start = p.kv_indptr[b];
+  const int kn = max(p.kv_indptr[b + 1] - kv_start, 0);
+  const int prefix = p.prefix_lens[b];
+  const int rows_total = q_len * p.group;
+  const int row0 = qblk * kRows;
+  if (row0 >= rows_total) return;
+
+  const bool idle = __builtin_amdgcn_readfirstlane(row0 + w * 32 >= rows_total ? 1 : 0) != 0;
+  const int qi_lo = row0 / p.group;
+  const int qi_hi = min(rows_total - 1, row0 + kRows - 1) / p.group;
+  int k_hi = p.is_cross ? kn : min(kn, prefix + qi_hi + 1);
+  int k_lo = (p.window > 0) ? max(0, prefix + qi_lo - p.window + 1) : 0;
+  k_lo &= ~(kBN - 1);
+  if (k_hi < k_lo) k_hi = k_lo;
+  if (p.n_ksplit > 1) {
+    const int all_tiles = (k_hi - k_lo + kBN - 1) / kBN;
+    const int share = (all_tiles + p.n_ksplit - 1) / p.n_ksplit * kBN;
+    k_lo = min(k_lo + split * share, k_hi);
+    k_hi = min(k_hi, k_lo + share);
+  }
+  const int n_tiles = (k_hi - k_lo + kBN - 1) / kBN;
+
+  // ---- this lane's row: Q operand, visibility bounds ---------------------------------------
+  bf16x8_t qreg[KSTEPS];
+  int row_lo, row_hi;
+  int w_lo_max = -0x7fffffff, w_hi_min = 0x7fffffff;
+  {
+    const int row = row0 + w * 32 + c32;
+    const bool valid = row < rows_total;
+    const int qi = valid ? row / p.group : 0;
+    const int hh = valid ? row - qi * p.group : 0;
+    const int64_t off = ((int64_t)(q_start + qi) * p.n_q + kvh * p.group + hh) * D;
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+      u32x4_t raw = {0u, 0u, 0u, 0u};
+      if (valid) raw = ld_global_b128(p.q + off + ks * 16 + h * 8);
+      qreg[ks] = as_bf16x8(raw);
+    }
+    const int qpos = prefix + qi;
+    int lo = (p.window > 0) ? qpos - p.window + 1 : 0;
+    int hi = min(p.is_cross ? kn - 1 : min(qpos, kn - 1), k_hi - 1);
+    if (valid) {
+      w_lo_max = lo;
+      w_hi_min = hi;
+    } else {
+      lo = 1;
+      hi = 0;
+    }
+    row_lo = lo;
+    row_hi = hi;
+  }
+#pragma unroll
+  for (int off = 1; off < kWave; off <<= 1) {
+    w_lo_max = max(w_lo_max, __shfl_xor(w_lo_max, off, kWave));
+    w_hi_min = min(w_hi_min, __shfl_xor(w_hi_min, off, kWave));
+  }
+  w_lo_max = __builtin_amdgcn_readfirstlane(w_lo_max);
+  w_hi_min = __builtin_amdgcn_readfirstlane(w_hi_min);
+
+  f32x16_t oacc[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) oacc[dt][i] = 0.f;
+  float m_run = kNegInf, l_run = 0.f, m_safe_run = 0.f;
+
+  // ---- moving tiles -------------------------------------------------------------------------
+  const uint32_t lds0 = (uint32_t)(uintptr_t)MSGL_LDS_PTR(unsigned char, smem);
+  const int32_t* idx_base = p.kv_indices + kv_start;
+  const unsigned char* k_src = reinterpret_cast<const unsigned char*>(p.k_cache + (int64_t)kvh * D);
+  const unsigned char* v_src = reinterpret_cast<const unsigned char*>(p.v_cache + (int64_t)kvh * D);
+  const uint32_t k_row_bytes = (uint32_t)p.k_stride0 * 2u;
+  const uint32_t v_row_bytes = (uint32_t)p.v_stride0 * 2u;
+  const uint32_t chunk_off = (uint32_t)(lane & 15) * 16u;
+  const int unit_key = w * UPW + 16 * (lane >> 4);  // + i for unit i of this wave
+  auto row_offset = [&](uint32_t slot_id, uint32_t row_bytes) -> OffT {
+    if constexpr (WIDE) return (uint64_t)slot_id * row_bytes + chunk_off;
+    else return __umul24(slot_id, row_bytes) + chunk_off;  // both below 2^24 here
+  };
+  // ring entry e of a wave = slot id of key (w UPW + e % UPW + 16 (e / UPW)) of the tile,
+  // e = 0 .. 4 UPW - 1; lanes past that repeat the entries
+  const uint32_t ring0 = (uint32_t)pp::kRingBase + (uint32_t)w * pp::kRingWave;
+  const int ring_key = w * UPW + (lane % UPW) + 16 * ((lane / UPW) & 3);
+  auto ring_fetch = [&](int t) {  // tile t of this block
+    const uint32_t off = (uint32_t)min(k_lo + t * kBN + ring_key, kn - 1) * 4u;
+    lds_direct_b32(lds0 + ring0 + (uint32_t)(t & (pp::kRingStages - 1)) * pp::kRingStage, idx_base, off);
+  };
+  auto ring_read = [&](int t, uint32_t (&ids)[UPW]) {
+    // read through an LDS pointer: a volatile read through a generic one would be a flat load,
+    // which waits for every vector-memory operation in flight
+    const volatile __attribute__((address_space(3))) uint32_t* r = MSGL_LDS_PTR(
+        const volatile uint32_t, smem + ring0 + (t & (pp::kRingStages - 1)) * pp::kRingStage + (lane >> 4) * (4 * UPW));
+#pragma unroll
+    for (int i = 0; i < UPW; ++i) ids[i] = min(r[i], p.max_slot);
+  };
+  uint32_t ids[UPW];  // slot ids of the tile whose K leaves in the next M phase
+  OffT v_off[UPW];    // V row offsets of the tile whose V leaves in the next M phase
+  auto k_stage_of = [](int t) { return (uint32_t)(t & 3) * kKStage; };
+  auto v_stage_of = [](int t) { return (uint32_t)pp::kVBase + (uint32_t)(t & 3) * kVStage; };
+  // The vector-memory part of M phase j in three pieces that ride along with its first slices:
+  // ids of tile j+6 requested; V(j+3) sent; K(j+4) sent and the V offsets of tile j+4 kept.
+  auto send_tiles = [&](int j, int piece) {
+    if (piece == 0) {
+      ring_fetch(j + 6);
+    } else if (piece == 1) {
+#pragma unroll
+      for (int i = 0; i < UPW; ++i)
+        lds_direct_b128(lds0 + v_stage_of(j + 3) + (uint32_t)(w * UPW + i) * kVUnit, v_src, v_off[i]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < UPW; ++i)
+        lds_direct_b128(lds0 + k_stage_of(j + 4) + (uint32_t)(w * UPW + i) * kKUnit, k_src,
+                        row_offset(ids[i], k_row_bytes));
+#pragma unroll
+      for (int i = 0; i < UPW; ++i) v_off[i] = row_offset(ids[i], v_row_bytes);
+    }
+  };
+  // end of M phase j: everything older than this phase's own ring fetch and moves has landed,
+  // among it the ring entries of tile j+5, which the next M phase turns into addresses
+  auto end_of_sends = [&](int j) {
+    wait_vm_at_most<2 * UPW + 1>();
+    ring_read(j + 5, ids);
+  };
+  auto slot_barrier = [&]() {
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  // per-lane LDS read offsets inside a stage (see prefill_tile_kernel)
+  const uint32_t k_lane = (uint32_t)(c32 & 15) * kKUnit + (uint32_t)(c32 >> 4) * 256u + (uint32_t)h * 16u;
+  const uint32_t v_lane = (uint32_t)(4 * h + ((lane & 15) >> 2)) * kVUnit +
+                          (uint32_t)((lane >> 4) & 1) * 32u + (uint32_t)(lane & 3) * 8u;
+
+  // S^T of one tile: s[kt][i] is key 32 kt + 8 (i / 4) + 4 h + i % 4, row c32
+  f32x16_t s[2];
+  bf16x8_t pb[2][2];  // P^T operands: [half][16 keys]
+  auto k_ops = [&](const unsigned char* ks, int kt, int first, bf16x8_t (&ops)[4]) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      ops[e] = as_bf16x8(*reinterpret_cast<const u32x4_t*>(ks + kt * 512 + (first + e) * 32));
+  };
+  auto v_ops = [&](const unsigned char* vs, int kt, int u, bf16x8_t (&ops)[4]) {
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      const u32x2_t lo = lds_read_tr16(vs + kt * 512 + u * 256 + dt * 64);
+      const u32x2_t hi = lds_read_tr16(vs + kt * 512 + u * 256 + dt * 64 + 8 * kVUnit);
+      ops[dt] = as_bf16x8(u32x4_t{lo[0], lo[1], hi[0], hi[1]});
+    }
+  };
+  auto pv4 = [&](const bf16x8_t& pw, const bf16x8_t (&ops)[4]) {
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) oacc[dt] = mfma_32x32x16(ops[dt], pw, oacc[dt]);
+  };
+  auto qk4 = [&](int kt, int first, const bf16x8_t (&ops)[4]) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) s[kt] = mfma_32x32x16(ops[e], qreg[first + e], s[kt]);
+  };
+  auto zero_scores = [&]() {
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) s[kt][i] = 0.f;
+  };
+  // Lane maximum of half kt of the scores, as two independent chains (a single chain would pay
+  // the full VALU latency per link: the partner wave issues no VALU work to fill the gaps).
+  auto half_max = [&](int kt) {
+    const f32x16_t& x = s[kt];
+    float m2[2];
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+      const int o = 8 * c;
+      float t = fmaxf(fmaxf(x[o], x[o + 1]), x[o + 2]);
+      t = fmaxf(fmaxf(t, x[o + 3]), x[o + 4]);
+      t = fmaxf(fmaxf(t, x[o + 5]), x[o + 6]);
+      m2[c] = fmaxf(t, x[o + 7]);
+    }
+    return fmaxf(m2[0], m2[1]);
+  };
+  float mx_lane = kNegInf;  // lane maximum of the raw scores of the tile in `s`
+  // M phase j: first the scores of tile j+1, then P V of tile j, with the lane maximum of the new
+  // scores taken in the shadow of the P V MFMAs.  The first slice's operands (`oa`: K(j+1), half
+  // 0, k-steps 0..3, or without QK: V(j), half 0, keys 0..15) were requested before the barrier
+  // (not so in the prologue's phase -1).  Every slice requests the operands of the next one
+  // first; the tile sends ride along with the first three slices.
+  auto m_phase = [&](int j, bf16x8_t (&oa)[4], auto with_pv, auto with_qk) {
+    constexpr bool PV = decltype(with_pv)::value, QK = decltype(with_qk)::value;
+    __builtin_amdgcn_s_setprio(MSGL_PP_PRIO_M);
+    const unsigned char* ks = smem + k_stage_of(j + 1) + k_lane;
+    const unsigned char* vs = smem + v_stage_of(j) + v_lane;
+    bf16x8_t ob[4];
+    // inside a slice: the LDS requests for the next slice first (they have the four MFMAs of this
+    // slice to arrive), then the MFMAs, whatever rides along in between
+#define reads_first(n_reads)                                  \
+  __builtin_amdgcn_sched_group_barrier(0x100, (n_reads), 0); \
+  __builtin_amdgcn_sched_group_barrier(0x008, 1, 0)
+    if constexpr (QK) {
+      if constexpr (!PV) k_ops(ks, 0, 0, oa);
+      zero_scores();
+      k_ops(ks, 0, 4, ob); qk4(0, 0, oa); send_tiles(j, 0); reads_first(4); __builtin_amdgcn_sched_barrier(0);
+      k_ops(ks, 1, 0, oa); qk4(0, 4, ob); send_tiles(j, 1); reads_first(4); __builtin_amdgcn_sched_barrier(0);
+      k_ops(ks, 1, 4, ob); qk4(1, 0, oa); send_tiles(j, 2); reads_first(4); __builtin_amdgcn_sched_barrier(0);
+      if constexpr (PV) v_ops(vs, 0, 0, oa);
+      qk4(1, 4, ob); if constexpr (PV) reads_first(8); __builtin_amdgcn_sched_barrier(0);
+    }
+    float mx0 = kNegInf;
+    if constexpr (PV) {
+      v_ops(vs, 0, 1, ob); pv4(pb[0][0], oa); if constexpr (QK) { mx0 = half_max(0); pin(mx0); } reads_first(8); __builtin_amdgcn_sched_barrier(0);
+      v_ops(vs, 1, 0, oa); pv4(pb[0][1], ob); reads_first(8); __builtin_amdgcn_sched_barrier(0);
+      v_ops(vs, 1, 1, ob); pv4(pb[1][0], oa); if constexpr (QK) { mx_lane = fmaxf(mx0, half_max(1)); pin(mx_lane); } reads_first(8); __builtin_amdgcn_sched_barrier(0);
+      pv4(pb[1][1], ob); __builtin_amdgcn_sched_barrier(0);
+    } else {
+      mx_lane = fmaxf(half_max(0), half_max(1));
+    }
+#undef reads_first
+    if constexpr (QK) end_of_sends(j);
+    __builtin_amdgcn_s_setprio(MSGL_PP_PRIO_V);
+  };
+  using Yes = std::true_type;
+  using No = std::false_type;
+
+  const bool general_scale = p.scale_log2e <= 0.f;  // the fast path needs a positive scale
+  // V phase j: P(j+1) from S(j+1) and its lane maxima, then the first operands of M phase j+1
+  auto v_phase = [&](int j, bf16x8_t (&oa)[4]) {
+    const int base = k_lo + (j + 1) * kBN;
+    float mul = p.scale_log2e;
+    if (general_scale || base < w_lo_max || base + kBN - 1 > w_hi_min) {
+      // boundary tile: scale and mask in place.  The empty volatile statement keeps this a
+      // branch: as selects it would put 100 more VALU instructions into every tile.
+      asm volatile("" ::: "memory");
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int key = base + 32 * kt + 8 * (i >> 2) + 4 * h + (i & 3);
+          const float x = s[kt][i] * p.scale_log2e;
+          s[kt][i] = (key < row_lo || key > row_hi) ? kNegInf : x;
+        }
+      mul = 1.0f;
+      mx_lane = fmaxf(half_max(0), half_max(1));
+    }
+    float mx = mx_lane;
+    float m_safe = m_safe_run, alpha = 1.0f;
+    // Usual case: no lane of the wave saw a score more than kLazy above its row's running max,
+    // so no row's max moves (both halves of a row sit in this wave).  Otherwise the cross-lane
+    // exchange, the new state and, where a max did move, the rescaling of O.
+    if (__any(mx * mul > m_run + kLazy)) {
+      const float m = wave_max_xor(mx * mul, 32);
+      const float m_old = m_run;
+      const float m_new = fmaxf(m_old, m);
+      const float m_use = (m_new - m_old > kLazy) ? m_new : m_old;
+      m_safe = (m_use == kNegInf) ? 0.f : m_use;
+      m_safe_run = m_safe;
+      alpha = fast_exp2(m_old - m_safe);
+      m_run = m_use;
+      if (__any(alpha != 1.0f)) {
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) oacc[dt][i] *= alpha;
+      }
+    }
+    float psum[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        u32x4_t pk;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float e0 = fast_exp2(__builtin_fmaf(s[kt][8 * u + 2 * e], mul, -m_safe));
+          const float e1 = fast_exp2(__builtin_fmaf(s[kt][8 * u + 2 * e + 1], mul, -m_safe));
+          const uint32_t pw = pack_bf16x2(e0, e1);
+          pk[e] = pw;
+          // row sum of the rounded weights, the ones that multiply V
+          psum[e] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, pw), kOnes, psum[e], false);
+        }
+        pb[kt][u] = as_bf16x8(pk);
+      }
+    l_run = l_run * alpha + ((psum[0] + psum[1]) + (psum[2] + psum[3]));
+    __builtin_amdgcn_sched_barrier(0);
+    // first operands of M phase j+1: its scores' if it computes any, else its P V's
+    if (j + 2 < n_tiles) k_ops(smem + k_stage_of(j + 2) + k_lane, 0, 0, oa);
+    else v_ops(smem + v_stage_of(j + 1) + v_lane, 0, 0, oa);
+  };
+
+  if (n_tiles > 0) {
+    // ---- prologue: K(0..2) and V(0..1) leave and are waited for; the ring holds tiles 3, 4 ---
+    {
+      uint32_t first[3][UPW];
+#pragma unroll
+      for (int t = 0; t < 3; ++t)
+#pragma unroll
+        for (int i = 0; i < UPW; ++i)
+          first[t][i] = min((uint32_t)idx_base[min(k_lo + t * kBN + unit_key + i, kn - 1)], p.max_slot);
+      ring_fetch(3);
+      ring_fetch(4);
+#pragma unroll
+      for (int t = 0; t < 3; ++t) {
+#pragma unroll
+        for (int i = 0; i < UPW; ++i) {
+          v_off[i] = row_offset(first[t][i], v_row_bytes);
+          lds_direct_b128(lds0 + k_stage_of(t) + (uint32_t)(w * UPW + i) * kKUnit, k_src,
+                          row_offset(first[t][i], k_row_bytes));
+          if (t < 2) lds_direct_b128(lds0 + v_stage_of(t) + (uint32_t)(w * UPW + i) * kVUnit, v_src, v_off[i]);
+        }
+      }
+      // v_off: tile 2, whose V leaves in M phase -1
+    }
+    wait_all_vm();
+    ring_read(3, ids);
+    __syncthreads();
+    const bool second = w >= 4;  // the group that runs one slot behind
+    if (idle) {
+      // the moves, waits and barriers of a computing wave of the same group, nothing else
+      if (second) slot_barrier();
+      for (int j = -1; j < n_tiles - 1; ++j) {
+#pragma unroll
+        for (int piece = 0; piece < 3; ++piece) send_tiles(j, piece);
+        end_of_sends(j);
+        slot_barrier();
+        slot_barrier();
+      }
+      wait_all_vm();
+      slot_barrier();
+      if (!second) slot_barrier();
+    } else {
+      bf16x8_t oa[4];
+      if (second) slot_barrier();
+      m_phase(-1, oa, No{}, Yes{});
+      slot_barrier();
+      v_phase(-1, oa);
+      slot_barrier();
+      for (int j = 0; j < n_tiles - 1; ++j) {
+        m_phase(j, oa, Yes{}, Yes{});
+        slot_barrier();
+        v_phase(j, oa);
+        slot_barrier();
+      }
+      m_phase(n_tiles - 1, oa, Yes{}, No{});
+      wait_all_vm();
+      slot_barrier();
+      if (!second) slot_barrier();
+    }
+    // every wave has passed its last read of the stages and every move has landed: the
+    // epilogue reuses the stages as its output staging area
+  }
+
+  // accumulator i of O^T tile dt is dim 32dt + 8(i/4) + 4h + i%4 of query row c32
+  float l = l_run;
+  l += __shfl_xor(l, 32, kWave);
+  const float inv = (l > 0.f) ? 1.0f / l : 0.f;
+  if (p.n_ksplit > 1) {
+    const int row = row0 + w * 32 + c32;
+    if (row < rows_total) {
+      const int qi = row / p.group;
+      const int hh = row - qi * p.group;
+      const int64_t at = (int64_t)split * p.part_rows + (int64_t)(q_start + qi) * p.n_q + kvh * p.group + hh;
+      if (h == 0) p.part_lse[at] = (l > 0.f) ? m_run + __log2f(l) : kNegInf;
+      float* dst = p.part_o + at * D + 4 * h;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+          f32x4_t v = {oacc[dt][4 * a] * inv, oacc[dt][4 * a + 1] * inv, oacc[dt][4 * a + 2] * inv,
+                       oacc[dt][4 * a + 3] * inv};
+          *reinterpret_cast<f32x4_t*>(dst + 32 * dt + 8 * a) = v;
+        }
+    }
+    return;
+  }
+  unsigned char* os = smem;
+  {
+    const int lrow = w * 32 + c32;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int a = 0; a < 4; ++a) {
+        u32x2_t wv;
+        wv[0] = pack_bf16x2(oacc[dt][4 * a] * inv, oacc[dt][4 * a + 1] * inv);
+        wv[1] = pack_bf16x2(oacc[dt][4 * a + 2] * inv, oacc[dt][4 * a + 3] * inv);
+        *reinterpret_cast<u32x2_t*>(os + (lrow * OROW + 32 * dt + 8 * a + 4 * h) * 2) = wv;
+      }
+  }
+  __syncthreads();
+  constexpr int ROWS_PER_PASS = NW * 4;
+  const int c = tid & 15;
+#pragma unroll 4
+  for (int pass = 0; pass < kRows / ROWS_PER_PASS; ++pass) {
+    const int lrow = pass * ROWS_PER_PASS + (tid >> 4);
+    const int row = row0 + lrow;
+    if (row < rows_total) {
+      const int qi = row / p.group;
+      const int hh = row - qi * p.group;
+      const u32x4_t v = *reinterpret_cast<const u32x4_t*>(os + (lrow * OROW + c * 8) * 2);
+      st_global_b128(p.out + ((int64_t)(q_start + qi) * p.n_q + kvh * p.group + hh) * D + c * 8, v);
+    }
+  }
+}
+
+
 // ---- merge of a key-split launch: one 32-lane group per (token, q head) row -----------------
 template <int D>
 __global__ __launch_bounds__(256) void prefill_merge_kernel(const float* __restrict__ part_o,
@@ -696,7 +1184,10 @@ int launch_prefill_tile(const PrefillArgs& a, hipStream_t stream) {
   const int rc = make_prefill_params(a, p, n_blocks, wide);
   if (rc != MSGL_OK || n_blocks == 0) return rc;
   const dim3 grid((unsigned)n_blocks);
-  if (tile_variant() == 1) {
+  if (tile_variant() == 3) {
+    if (wide) hipLaunchKernelGGL((prefill_pingpong_kernel<true>), grid, dim3(512), 0, stream, p);
+    else hipLaunchKernelGGL((prefill_pingpong_kernel<false>), grid, dim3(512), 0, stream, p);
+  } else if (tile_variant() == 1) {
     if (wide) hipLaunchKernelGGL((prefill_tile_kernel<128, 2, 4, true>), grid, dim3(256), 0, stream, p);
     else hipLaunchKernelGGL((prefill_tile_kernel<128, 2, 4, false>), grid, dim3(256), 0, stream, p);
   } else {

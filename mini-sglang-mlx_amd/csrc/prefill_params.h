@@ -18,6 +18,7 @@ struct PrefillParams {
   int32_t n_qblk, n_pairs;  // q blocks per (request, kv head); batch * n_kv
   int32_t max_len_extend, is_cross, window;
   float scale_log2e;
+  uint32_t max_slot;  // num_slots - 1: slot ids are clamped to it before they become addresses
   // key splits: each workgroup takes one contiguous share of its rows' visible keys
   // and leaves a normalised fp32 partial and a base-2 log-sum-exp per row for the merge kernel
   int32_t n_ksplit;
@@ -111,6 +112,7 @@ inline int make_prefill_params(const PrefillArgs& a, PrefillParams& p, int64_t& 
   p.is_cross = a.is_cross;
   p.window = a.window;
   p.scale_log2e = a.sm_scale * 1.4426950408889634f;
+  p.max_slot = (uint32_t)(a.num_slots > 0 ? a.num_slots - 1 : 0);
   p.n_ksplit = a.key_splits > 1 ? a.key_splits : 1;
   p.part_rows = a.total_q * a.n_q;
   p.part_o = static_cast<float*>(a.workspace);

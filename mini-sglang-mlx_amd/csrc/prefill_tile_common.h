@@ -25,6 +25,13 @@ __device__ __forceinline__ void lds_direct_b128(uint32_t lds_addr, const void* s
                : "s"(lds_addr), "v"(a)
                : "memory");
 }
+// 64 lanes x 4 bytes: lane l's dword at `saddr + voff` lands at LDS byte lds_addr + 4 l.
+__device__ __forceinline__ void lds_direct_b32(uint32_t lds_addr, const void* saddr, uint32_t voff) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
+               :
+               : "s"(lds_addr), "v"(voff), "s"(saddr)
+               : "memory");
+}
 // s_waitcnt vmcnt(0) (expcnt and lgkmcnt fields left at their maxima).  Issued through the
 // builtin so that the compiler's own wait bookkeeping sees it.
 __device__ __forceinline__ void wait_all_vm() {
