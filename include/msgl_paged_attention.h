@@ -270,8 +270,10 @@ MSGL_API int msgl_gdn_state_inplace(const void* q, const void* k, const void* v,
  *   MSGL_TUNE_SEGMENTS       segments the split-K kernel cuts the visible token stream into
  *   MSGL_TUNE_MIN_SEGMENT    smallest segment length in tokens (multiple of 64)
  *   MSGL_TUNE_SMALLQ_MAXCOLS largest q_len*group routed to the split-K kernel
- *   MSGL_TUNE_PREFILL_VARIANT tiling of the head_dim 128 MFMA kernel (0: 8 waves x 32 rows,
- *                            1: 4 x 64); 2: head_dim 256 through split-K in query chunks
+ *   MSGL_TUNE_PREFILL_VARIANT head_dim 128 MFMA kernel: 0 the ping-pong kernel (8 waves x 32 rows,
+ *                            the two waves of a SIMD alternate between MFMA and softmax phases),
+ *                            3 the fused kernel it replaced (8 x 32), 1 the fused kernel with
+ *                            4 waves x 64 rows; 2: head_dim 256 through split-K in query chunks
  *   MSGL_TUNE_SPLITKV_WAVES  most waves (adjacent kv heads) per split-K workgroup: 1, 2, 4, 8
  *                            (0 restores the default, 4)
  *   MSGL_TUNE_GDN_ROWS       state rows per 16-lane group of the gdn_state kernel: 1, 2, 4

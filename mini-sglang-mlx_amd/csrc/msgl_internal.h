@@ -78,9 +78,9 @@ struct PrefillArgs {
 int launch_prefill_tile(const PrefillArgs& a, hipStream_t stream);     // head_dim 128
 // ---- paged_prefill_d256.hip ----------------------------------------------------------
 int launch_prefill_tile256(const PrefillArgs& a, hipStream_t stream);  // head_dim 256
-// benchmarking switch: tiling of the head_dim 128 kernel (0: 8 waves x 32 rows, 1: 4 waves x
-// 64 rows; both cover 256 rows per workgroup); 2 sends head_dim 256 through the split-K
-// kernel in chunks of queries instead of its tile kernel
+// benchmarking switch: head_dim 128 kernel (0: ping-pong kernel, 3: fused kernel with 8 waves x
+// 32 rows, 1: fused kernel with 4 waves x 64 rows; all cover 256 rows per workgroup); 2 sends
+// head_dim 256 through the split-K kernel in chunks of queries instead of its tile kernel
 int tile_variant();
 void set_tile_variant(int v);
 

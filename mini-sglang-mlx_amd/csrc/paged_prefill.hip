@@ -642,15 +642,18 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
 //   w >= 4   -      M(-1)   V(-1)   M(0)    V(0)
 //
 // Tiles: K(t) and V(t) live in stage t % 4 of four K and four V stages.  M phase j, whose wave
-// has issue slots to spare between its MFMAs, also sends K(j+4) and V(j+3) on their way (each
-// wave its two units of each) and, at its end, waits for what it sent in M phase j-1, so a tile
-// is in flight for two slots and has been published by a barrier a full slot before its first
-// reader asks for operands.  The slot ids of a tile travel through a small LDS ring of the
-// wave's own (one dword LDS-direct load per tile, two M phases ahead; read back into registers
-// at the end of the M phase before the one that uses them), which keeps every vector-memory
-// operation of the loop out of the compiler's wait bookkeeping: the only vector-memory wait in
-// the loop is the counted one at the end of an M phase.  Order of issue inside an M phase:
-// [ring fetch, 4 moves].
+// has issue slots to spare between its MFMAs, also sends K(j+4) and V(j+2) on their way (each
+// wave its two units of each) and, before the barrier that ends its slot, waits for what it sent
+// in M phase j-1: a tile is in flight for two slots and has been published by a barrier before
+// its first reader asks for operands.  A stage is refilled only after a barrier that every
+// reader of its previous tile has passed with its reads done: K(j) is read by the score slices
+// of M phase j-1, which precede that phase's barrier, and V(j-2) by M phase j-2, two phases back
+// (an M phase passes its barrier before its last P V slices, so "one phase back" would not do).
+// The slot ids of a tile travel through a small LDS ring of the wave's own (one dword
+// LDS-direct load per tile, two M phases ahead; read back into registers at the barrier of the
+// M phase before the one that uses them), which keeps every vector-memory operation of the loop
+// out of the compiler's wait bookkeeping: the only vector-memory wait in the loop is the counted
+// one before an M phase's barrier.  Order of issue inside an M phase: [ring fetch, 4 moves].
 #ifndef MSGL_PP_PRIO_M
 #define MSGL_PP_PRIO_M 3
 #endif
@@ -665,6 +668,21 @@ constexpr int kRingStage = 256;  // one dword per lane
 constexpr int kRingStages = 4;
 constexpr int kRingWave = kRingStages * kRingStage;
 constexpr int kSmem = kRingBase + 8 * kRingWave;
+// LDS operands of a slice of four MFMAs are requested this many slices ahead (two measured no
+// faster than one and costs 16 more registers)
+#ifndef MSGL_PP_AHEAD
+#define MSGL_PP_AHEAD 1
+#endif
+constexpr int kAhead = MSGL_PP_AHEAD;
+// An M phase passes the barrier that ends its slot this many slices before its last one: the
+// partner wave needs a few hundred cycles from the barrier to its first MFMA, and the matrix
+// pipe would idle for them.
+#ifndef MSGL_PP_HANDOFF
+#define MSGL_PP_HANDOFF 1
+#endif
+constexpr int kHandoff = MSGL_PP_HANDOFF;
+static_assert(kHandoff >= 0 && kHandoff <= 2, "the sends of a phase must have left before its barrier");
+constexpr int kOperandBuffers = kAhead + 1;
 }  // namespace pp
 
 template <bool WIDE>
@@ -807,25 +825,29 @@ __global__ __launch_bounds__(512) void prefill_pingpong_kernel(PrefillParams p) 
     for (int i = 0; i < UPW; ++i) ids[i] = min(r[i], p.max_slot);
   };
   uint32_t ids[UPW];  // slot ids of the tile whose K leaves in the next M phase
-  OffT v_off[UPW];    // V row offsets of the tile whose V leaves in the next M phase
+  OffT v_off[UPW];       // V row offsets of the tile whose V leaves in the next M phase
+  OffT v_off_then[UPW];  // ... and of the tile whose V leaves in the one after
   auto k_stage_of = [](int t) { return (uint32_t)(t & 3) * kKStage; };
   auto v_stage_of = [](int t) { return (uint32_t)pp::kVBase + (uint32_t)(t & 3) * kVStage; };
   // The vector-memory part of M phase j in three pieces that ride along with its first slices:
-  // ids of tile j+6 requested; V(j+3) sent; K(j+4) sent and the V offsets of tile j+4 kept.
+  // ids of tile j+6 requested; V(j+2) sent; K(j+4) sent and the V offsets of tile j+4 kept.
   auto send_tiles = [&](int j, int piece) {
     if (piece == 0) {
       ring_fetch(j + 6);
     } else if (piece == 1) {
 #pragma unroll
       for (int i = 0; i < UPW; ++i)
-        lds_direct_b128(lds0 + v_stage_of(j + 3) + (uint32_t)(w * UPW + i) * kVUnit, v_src, v_off[i]);
+        lds_direct_b128(lds0 + v_stage_of(j + 2) + (uint32_t)(w * UPW + i) * kVUnit, v_src, v_off[i]);
     } else {
 #pragma unroll
       for (int i = 0; i < UPW; ++i)
         lds_direct_b128(lds0 + k_stage_of(j + 4) + (uint32_t)(w * UPW + i) * kKUnit, k_src,
                         row_offset(ids[i], k_row_bytes));
 #pragma unroll
-      for (int i = 0; i < UPW; ++i) v_off[i] = row_offset(ids[i], v_row_bytes);
+      for (int i = 0; i < UPW; ++i) {
+        v_off[i] = v_off_then[i];
+        v_off_then[i] = row_offset(ids[i], v_row_bytes);
+      }
     }
   };
   // end of M phase j: everything older than this phase's own ring fetch and moves has landed,
@@ -890,51 +912,81 @@ __global__ __launch_bounds__(512) void prefill_pingpong_kernel(PrefillParams p) 
     }
     return fmaxf(m2[0], m2[1]);
   };
-  float mx_lane = kNegInf;  // lane maximum of the raw scores of the tile in `s`
-  // M phase j: first the scores of tile j+1, then P V of tile j, with the lane maximum of the new
-  // scores taken in the shadow of the P V MFMAs.  The first slice's operands (`oa`: K(j+1), half
-  // 0, k-steps 0..3, or without QK: V(j), half 0, keys 0..15) were requested before the barrier
-  // (not so in the prologue's phase -1).  Every slice requests the operands of the next one
-  // first; the tile sends ride along with the first three slices.
-  auto m_phase = [&](int j, bf16x8_t (&oa)[4], auto with_pv, auto with_qk) {
+  // M phase j: first the scores of tile j+1, then P V of tile j.  Eight slices of four MFMAs; the
+  // operands of a slice are requested kAhead slices ahead into one of kAhead + 1 operand
+  // buffers, those of the first slice(s) before the barrier (in the first and the last phase: at
+  // its start).  The tile sends ride along with the first three slices; the barrier that ends
+  // the phase's slot comes kHandoff slices before the end.  Nothing else rides along: the wave's
+  // issue slots between MFMAs are taken by the LDS requests and their waits (measured: with the
+  // row maxima computed here instead of in the V phase the kernel is 2 % slower).
+  auto m_phase = [&](int j, bf16x8_t (&o)[pp::kOperandBuffers][4], auto with_pv, auto with_qk) {
     constexpr bool PV = decltype(with_pv)::value, QK = decltype(with_qk)::value;
+    constexpr int NS = 4 * ((PV ? 1 : 0) + (QK ? 1 : 0));  // slices of four MFMAs
     __builtin_amdgcn_s_setprio(MSGL_PP_PRIO_M);
     const unsigned char* ks = smem + k_stage_of(j + 1) + k_lane;
     const unsigned char* vs = smem + v_stage_of(j) + v_lane;
-    bf16x8_t ob[4];
-    // inside a slice: the LDS requests for the next slice first (they have the four MFMAs of this
-    // slice to arrive), then the MFMAs, whatever rides along in between
-#define reads_first(n_reads)                                  \
-  __builtin_amdgcn_sched_group_barrier(0x100, (n_reads), 0); \
-  __builtin_amdgcn_sched_group_barrier(0x008, 1, 0)
-    if constexpr (QK) {
-      if constexpr (!PV) k_ops(ks, 0, 0, oa);
-      zero_scores();
-      k_ops(ks, 0, 4, ob); qk4(0, 0, oa); send_tiles(j, 0); reads_first(4); __builtin_amdgcn_sched_barrier(0);
-      k_ops(ks, 1, 0, oa); qk4(0, 4, ob); send_tiles(j, 1); reads_first(4); __builtin_amdgcn_sched_barrier(0);
-      k_ops(ks, 1, 4, ob); qk4(1, 0, oa); send_tiles(j, 2); reads_first(4); __builtin_amdgcn_sched_barrier(0);
-      if constexpr (PV) v_ops(vs, 0, 0, oa);
-      qk4(1, 4, ob); if constexpr (PV) reads_first(8); __builtin_amdgcn_sched_barrier(0);
+    // slice i: scores (half i / 2, k-steps 4 (i % 2) ..) while i < 4 and QK, else P V
+    auto request = [&](auto ic) {
+      constexpr int i = decltype(ic)::value;
+      if constexpr (i < NS) {
+        if constexpr (QK && i < 4) k_ops(ks, i >> 1, (i & 1) * 4, o[i % pp::kOperandBuffers]);
+        else v_ops(vs, (i - (QK ? 4 : 0)) >> 1, (i - (QK ? 4 : 0)) & 1, o[i % pp::kOperandBuffers]);
+      }
+    };
+    auto slice = [&](auto ic) {
+      constexpr int i = decltype(ic)::value;
+      if constexpr (QK && pp::kHandoff > 0 && i == NS - pp::kHandoff) {
+        end_of_sends(j);
+        slot_barrier();
+      }
+      request(std::integral_constant<int, i + pp::kAhead>{});
+      if constexpr (QK && i < 4) {
+        qk4(i >> 1, (i & 1) * 4, o[i % pp::kOperandBuffers]);
+        if constexpr (NS == 8) {
+          if constexpr (i < 3) send_tiles(j, i);
+        } else {  // four slices: everything has to leave before the barrier
+          if constexpr (i == 0) { send_tiles(j, 0); send_tiles(j, 1); }
+          if constexpr (i == 1) send_tiles(j, 2);
+        }
+      } else {
+        constexpr int r = i - (QK ? 4 : 0);
+        pv4(pb[r >> 1][r & 1], o[i % pp::kOperandBuffers]);
+      }
+      // the LDS requests first, then the MFMAs and whatever rides along
+      if constexpr (i + pp::kAhead < NS) {
+        if constexpr (QK && i + pp::kAhead < 4) __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+        else __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    if constexpr (!(QK && PV)) {  // the first and the last phase: nothing was requested ahead
+      request(std::integral_constant<int, 0>{});
+      if constexpr (pp::kAhead > 1) request(std::integral_constant<int, 1>{});
     }
-    float mx0 = kNegInf;
-    if constexpr (PV) {
-      v_ops(vs, 0, 1, ob); pv4(pb[0][0], oa); if constexpr (QK) { mx0 = half_max(0); pin(mx0); } reads_first(8); __builtin_amdgcn_sched_barrier(0);
-      v_ops(vs, 1, 0, oa); pv4(pb[0][1], ob); reads_first(8); __builtin_amdgcn_sched_barrier(0);
-      v_ops(vs, 1, 1, ob); pv4(pb[1][0], oa); if constexpr (QK) { mx_lane = fmaxf(mx0, half_max(1)); pin(mx_lane); } reads_first(8); __builtin_amdgcn_sched_barrier(0);
-      pv4(pb[1][1], ob); __builtin_amdgcn_sched_barrier(0);
-    } else {
-      mx_lane = fmaxf(half_max(0), half_max(1));
+    if constexpr (QK) zero_scores();
+    slice(std::integral_constant<int, 0>{});
+    slice(std::integral_constant<int, 1>{});
+    slice(std::integral_constant<int, 2>{});
+    slice(std::integral_constant<int, 3>{});
+    if constexpr (NS == 8) {
+      slice(std::integral_constant<int, 4>{});
+      slice(std::integral_constant<int, 5>{});
+      slice(std::integral_constant<int, 6>{});
+      slice(std::integral_constant<int, 7>{});
     }
-#undef reads_first
-    if constexpr (QK) end_of_sends(j);
+    if constexpr (QK && pp::kHandoff == 0) {
+      end_of_sends(j);
+      slot_barrier();
+    }
     __builtin_amdgcn_s_setprio(MSGL_PP_PRIO_V);
   };
   using Yes = std::true_type;
   using No = std::false_type;
 
   const bool general_scale = p.scale_log2e <= 0.f;  // the fast path needs a positive scale
-  // V phase j: P(j+1) from S(j+1) and its lane maxima, then the first operands of M phase j+1
-  auto v_phase = [&](int j, bf16x8_t (&oa)[4]) {
+  // V phase j: P(j+1) from S(j+1), then the first operands of M phase j+1
+  auto v_phase = [&](int j, bf16x8_t (&o)[pp::kOperandBuffers][4]) {
     const int base = k_lo + (j + 1) * kBN;
     float mul = p.scale_log2e;
     if (general_scale || base < w_lo_max || base + kBN - 1 > w_hi_min) {
@@ -950,9 +1002,8 @@ __global__ __launch_bounds__(512) void prefill_pingpong_kernel(PrefillParams p) 
           s[kt][i] = (key < row_lo || key > row_hi) ? kNegInf : x;
         }
       mul = 1.0f;
-      mx_lane = fmaxf(half_max(0), half_max(1));
     }
-    float mx = mx_lane;
+    const float mx = fmaxf(half_max(0), half_max(1));
     float m_safe = m_safe_run, alpha = 1.0f;
     // Usual case: no lane of the wave saw a score more than kLazy above its row's running max,
     // so no row's max moves (both halves of a row sit in this wave).  Otherwise the cross-lane
@@ -992,13 +1043,18 @@ __global__ __launch_bounds__(512) void prefill_pingpong_kernel(PrefillParams p) 
       }
     l_run = l_run * alpha + ((psum[0] + psum[1]) + (psum[2] + psum[3]));
     __builtin_amdgcn_sched_barrier(0);
-    // first operands of M phase j+1: its scores' if it computes any, else its P V's
-    if (j + 2 < n_tiles) k_ops(smem + k_stage_of(j + 2) + k_lane, 0, 0, oa);
-    else v_ops(smem + v_stage_of(j + 1) + v_lane, 0, 0, oa);
+    // operands of the first slice(s) of M phase j+1: its scores' if it computes any, else
+    // its P V's
+    if (j + 2 < n_tiles) {
+      k_ops(smem + k_stage_of(j + 2) + k_lane, 0, 0, o[0]);
+      if constexpr (pp::kAhead > 1) k_ops(smem + k_stage_of(j + 2) + k_lane, 0, 4, o[1]);
+    }
+    // (the last phase, P V only, asks for its operands itself: the V tile it reads may only have
+    // been published by the barrier that precedes it)
   };
 
   if (n_tiles > 0) {
-    // ---- prologue: K(0..2) and V(0..1) leave and are waited for; the ring holds tiles 3, 4 ---
+    // ---- prologue: K(0..2) and V(0) leave and are waited for; the ring holds tiles 3, 4 ------
     {
       uint32_t first[3][UPW];
 #pragma unroll
@@ -1012,13 +1068,14 @@ __global__ __launch_bounds__(512) void prefill_pingpong_kernel(PrefillParams p) 
       for (int t = 0; t < 3; ++t) {
 #pragma unroll
         for (int i = 0; i < UPW; ++i) {
-          v_off[i] = row_offset(first[t][i], v_row_bytes);
+          const OffT vo = row_offset(first[t][i], v_row_bytes);
           lds_direct_b128(lds0 + k_stage_of(t) + (uint32_t)(w * UPW + i) * kKUnit, k_src,
                           row_offset(first[t][i], k_row_bytes));
-          if (t < 2) lds_direct_b128(lds0 + v_stage_of(t) + (uint32_t)(w * UPW + i) * kVUnit, v_src, v_off[i]);
+          if (t == 0) lds_direct_b128(lds0 + v_stage_of(t) + (uint32_t)(w * UPW + i) * kVUnit, v_src, vo);
+          if (t == 1) v_off[i] = vo;       // leaves in M phase -1
+          if (t == 2) v_off_then[i] = vo;  // leaves in M phase 0
         }
       }
-      // v_off: tile 2, whose V leaves in M phase -1
     }
     wait_all_vm();
     ring_read(3, ids);
@@ -1038,15 +1095,13 @@ __global__ __launch_bounds__(512) void prefill_pingpong_kernel(PrefillParams p) 
       slot_barrier();
       if (!second) slot_barrier();
     } else {
-      bf16x8_t oa[4];
+      bf16x8_t oa[pp::kOperandBuffers][4];
       if (second) slot_barrier();
-      m_phase(-1, oa, No{}, Yes{});
-      slot_barrier();
+      m_phase(-1, oa, No{}, Yes{});  // with its barrier
       v_phase(-1, oa);
       slot_barrier();
       for (int j = 0; j < n_tiles - 1; ++j) {
-        m_phase(j, oa, Yes{}, Yes{});
-        slot_barrier();
+        m_phase(j, oa, Yes{}, Yes{});  // with its barrier
         v_phase(j, oa);
         slot_barrier();
       }
@@ -1184,15 +1239,15 @@ int launch_prefill_tile(const PrefillArgs& a, hipStream_t stream) {
   const int rc = make_prefill_params(a, p, n_blocks, wide);
   if (rc != MSGL_OK || n_blocks == 0) return rc;
   const dim3 grid((unsigned)n_blocks);
-  if (tile_variant() == 3) {
-    if (wide) hipLaunchKernelGGL((prefill_pingpong_kernel<true>), grid, dim3(512), 0, stream, p);
-    else hipLaunchKernelGGL((prefill_pingpong_kernel<false>), grid, dim3(512), 0, stream, p);
-  } else if (tile_variant() == 1) {
+  if (tile_variant() == 1) {
     if (wide) hipLaunchKernelGGL((prefill_tile_kernel<128, 2, 4, true>), grid, dim3(256), 0, stream, p);
     else hipLaunchKernelGGL((prefill_tile_kernel<128, 2, 4, false>), grid, dim3(256), 0, stream, p);
-  } else {
+  } else if (tile_variant() == 3) {
     if (wide) hipLaunchKernelGGL((prefill_tile_kernel<128, 1, 8, true>), grid, dim3(512), 0, stream, p);
     else hipLaunchKernelGGL((prefill_tile_kernel<128, 1, 8, false>), grid, dim3(512), 0, stream, p);
+  } else {
+    if (wide) hipLaunchKernelGGL((prefill_pingpong_kernel<true>), grid, dim3(512), 0, stream, p);
+    else hipLaunchKernelGGL((prefill_pingpong_kernel<false>), grid, dim3(512), 0, stream, p);
   }
   const int launched = check_launch();
   if (launched != MSGL_OK || p.n_ksplit == 1) return launched;

@@ -62,9 +62,9 @@ def test_store_then_prefill_reaches_written_slots(gpu):
                                expected_weights(q_len, 0, False, 0), rtol=1e-3, atol=1e-3)
 
 
-@pytest.fixture(params=[0, 1, 3], ids=["8x32rows", "4x64rows", "pingpong"])
+@pytest.fixture(params=[0, 1, 3], ids=["pingpong", "4x64rows", "8x32rows"])
 def tile_variant(request):
-    """Both tilings of the MFMA kernel are product code; each is checked."""
+    """The ping-pong kernel (default) and both tilings of the fused kernel are product code; each is checked."""
     from mini_sglang_amd_kernel import _lib
 
     _lib.set_tuning(_lib.TUNE_PREFILL_VARIANT, request.param)
