@@ -925,45 +925,51 @@ __global__ __launch_bounds__(512) void prefill_pingpong_kernel(PrefillParams p) 
     __builtin_amdgcn_s_setprio(MSGL_PP_PRIO_M);
     const unsigned char* ks = smem + k_stage_of(j + 1) + k_lane;
     const unsigned char* vs = smem + v_stage_of(j) + v_lane;
-    // slice i: scores (half i / 2, k-steps 4 (i % 2) ..) while i < 4 and QK, else P V
+    // Slice i is a score slice (half t / 2, k-steps 4 (t % 2) ..) or a P V slice (half t / 2, keys
+    // 16 (t % 2) ..), t = i % 4; a full phase runs its four score slices first.  (Alternating the
+    // two kinds, which spreads the transposing V reads over the phase, measured 2-5 % slower.)
     auto request = [&](auto ic) {
       constexpr int i = decltype(ic)::value;
       if constexpr (i < NS) {
-        if constexpr (QK && i < 4) k_ops(ks, i >> 1, (i & 1) * 4, o[i % pp::kOperandBuffers]);
-        else v_ops(vs, (i - (QK ? 4 : 0)) >> 1, (i - (QK ? 4 : 0)) & 1, o[i % pp::kOperandBuffers]);
+        constexpr bool is_qk = QK && (!PV || i < 4);
+        constexpr int t = i % 4;
+        if constexpr (is_qk) k_ops(ks, t >> 1, (t & 1) * 4, o[i % pp::kOperandBuffers]);
+        else v_ops(vs, t >> 1, t & 1, o[i % pp::kOperandBuffers]);
       }
     };
     auto slice = [&](auto ic) {
       constexpr int i = decltype(ic)::value;
+      constexpr bool is_qk = QK && (!PV || i < 4);
+      constexpr int t = i % 4;
       if constexpr (QK && pp::kHandoff > 0 && i == NS - pp::kHandoff) {
         end_of_sends(j);
         slot_barrier();
       }
       request(std::integral_constant<int, i + pp::kAhead>{});
-      if constexpr (QK && i < 4) {
-        qk4(i >> 1, (i & 1) * 4, o[i % pp::kOperandBuffers]);
+      if constexpr (is_qk) qk4(t >> 1, (t & 1) * 4, o[i % pp::kOperandBuffers]);
+      else pv4(pb[t >> 1][t & 1], o[i % pp::kOperandBuffers]);
+      if constexpr (QK) {  // the sends: all of them before the barrier
         if constexpr (NS == 8) {
           if constexpr (i < 3) send_tiles(j, i);
-        } else {  // four slices: everything has to leave before the barrier
+        } else {
           if constexpr (i == 0) { send_tiles(j, 0); send_tiles(j, 1); }
           if constexpr (i == 1) send_tiles(j, 2);
         }
-      } else {
-        constexpr int r = i - (QK ? 4 : 0);
-        pv4(pb[r >> 1][r & 1], o[i % pp::kOperandBuffers]);
       }
       // the LDS requests first, then the MFMAs and whatever rides along
       if constexpr (i + pp::kAhead < NS) {
-        if constexpr (QK && i + pp::kAhead < 4) __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+        constexpr int i2 = i + pp::kAhead;
+        constexpr bool next_qk = QK && (!PV || i2 < 4);
+        if constexpr (next_qk) __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
         else __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
       }
       __builtin_amdgcn_sched_barrier(0);
     };
-    if constexpr (!(QK && PV)) {  // the first and the last phase: nothing was requested ahead
-      request(std::integral_constant<int, 0>{});
-      if constexpr (pp::kAhead > 1) request(std::integral_constant<int, 1>{});
-    }
+    // Slice 0's operands were requested before the barrier in a full phase (the V tile may only
+    // just have been published, so nothing of it is asked for ahead of the barrier).
+    if constexpr (!(QK && PV)) request(std::integral_constant<int, 0>{});
+    if constexpr (pp::kAhead > 1) request(std::integral_constant<int, 1>{});
     if constexpr (QK) zero_scores();
     slice(std::integral_constant<int, 0>{});
     slice(std::integral_constant<int, 1>{});
@@ -1047,7 +1053,6 @@ __global__ __launch_bounds__(512) void prefill_pingpong_kernel(PrefillParams p) 
     // its P V's
     if (j + 2 < n_tiles) {
       k_ops(smem + k_stage_of(j + 2) + k_lane, 0, 0, o[0]);
-      if constexpr (pp::kAhead > 1) k_ops(smem + k_stage_of(j + 2) + k_lane, 0, 4, o[1]);
     }
     // (the last phase, P V only, asks for its operands itself: the V tile it reads may only have
     // been published by the barrier that precedes it)
