@@ -8,8 +8,8 @@
 //
 // Work decomposition
 //   The visible keys of all requests, in CSR order, form one token stream.  It is cut
-//   into `n_seg` equal segments (the count is chosen on the host: one workgroup per CU,
-//   all resident at once, one round, no tail; the HBM system, not the CUs, is the limit).
+//   into `n_seg` equal segments (the count is chosen on the host: workgroups for 13 of every
+//   16 CUs, all resident at once, one round, no tail; the HBM system, not the CUs, is the limit).
 //   A workgroup owns one segment and `nwh` adjacent kv heads, one wave64 per head; all
 //   waves walk the same tokens, so the workgroup touches nwh*256-byte stretches of every
 //   slot row together.  A wave holds up to two tiles of 16 columns; shapes with more
@@ -647,8 +647,12 @@ int splitkv_default_segments(int64_t total_kv, int64_t n_kv, int64_t head_dim, i
   const int nwh = nwh_for(n_kv, nct, head_dim);
   const int waves = nwh * col_split(nct, head_dim).col_waves;
   const int64_t head_groups = n_kv / nwh;
-  // one workgroup per CU; small workgroups are doubled up until a CU holds four waves
-  const int64_t blocks = (int64_t)device_cus() * (waves >= 4 ? 1 : 4 / waves);
+  // Workgroups for 13 of every 16 CUs, at most one per CU (small workgroups are doubled up until
+  // a CU holds four waves): the memory system is saturated well before every CU streams, and
+  // fewer, longer segments mean fewer partials and fewer request boundaries inside a segment.
+  // Measured at 256 CUs, segments per head group 80 .. 128: fastest at 96 .. 112 on every
+  // benchmark shape (1-2 % under 128), slower again below 88.
+  const int64_t blocks = (int64_t)device_cus() * 13 / 16 * (waves >= 4 ? 1 : 4 / waves);
   int64_t n_seg = blocks / head_groups;
   const int64_t by_len = (total_kv + min_seg - 1) / min_seg;
   if (n_seg > by_len) n_seg = by_len;
