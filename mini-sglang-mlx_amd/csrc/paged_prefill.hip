@@ -193,9 +193,11 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
   const uint32_t v_row_bytes = (uint32_t)p.v_stride0 * 2u;
   const uint32_t chunk_off = (uint32_t)(lane & 15) * 16u;
   const int unit_key = w * UPW + 16 * (lane >> 4);  // + i for unit i of this wave
+  // slot ids are clamped to the pool before they become addresses
   auto row_offset = [&](int32_t slot_id, uint32_t row_bytes) -> OffT {
-    if constexpr (WIDE) return (uint64_t)(uint32_t)slot_id * row_bytes + chunk_off;
-    else return __umul24((uint32_t)slot_id, row_bytes) + chunk_off;  // both below 2^24 here
+    const uint32_t id = min((uint32_t)slot_id, p.max_slot);
+    if constexpr (WIDE) return (uint64_t)id * row_bytes + chunk_off;
+    else return __umul24(id, row_bytes) + chunk_off;  // both below 2^24 here
   };
   int32_t slot[UPW];  // slot ids of the tile whose K moves next, fetched one iteration ahead
   OffT k_off[UPW];    // K row offsets of that tile

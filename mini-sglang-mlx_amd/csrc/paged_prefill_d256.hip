@@ -204,7 +204,10 @@ __global__ __launch_bounds__(kNW * 64) void prefill_tile256_kernel(PrefillParams
     static_assert(N >= 0 && N < 16, "low bits of vmcnt only");
     asm volatile("s_waitcnt vmcnt(%1)" : "+v"(sl) : "n"(N) : "memory");
   };
+  // slot ids are clamped to the pool before they become addresses: an id that is out of range
+  // (or stale) then reads a wrong row instead of faulting
   auto lane_offset = [&](uint32_t slot, uint32_t row_bytes) -> OffT {
+    slot = min(slot, p.max_slot);
     if constexpr (WIDE) return (uint64_t)slot * row_bytes + chunk_off;
     else return __umul24(slot, row_bytes) + chunk_off;  // both factors below 2^24 here
   };

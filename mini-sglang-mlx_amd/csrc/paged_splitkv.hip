@@ -67,6 +67,7 @@ struct SplitKvParams {
   int32_t f16;             // elements are IEEE half instead of bf16
   int32_t is_cross, window;
   int32_t wide;  // pool byte offsets need 64 bits
+  uint32_t max_slot;  // num_slots - 1: slot ids are clamped to it before they become addresses
   float scale_log2e;
 };
 
@@ -275,8 +276,8 @@ __global__ __launch_bounds__(64 * NW, ((D == 128 && NCT == 1) ? 2 : 1)) void spl
 
     // slot ids of the two K rows this lane loads in a 32-token tile starting at tb
     auto load_idx = [&](int tb, int& s0, int& s1) {
-      s0 = idx_base[min(tb + t16, last_tok)];
-      s1 = idx_base[min(tb + 16 + t16, last_tok)];
+      s0 = (int)min((uint32_t)idx_base[min(tb + t16, last_tok)], p.max_slot);
+      s1 = (int)min((uint32_t)idx_base[min(tb + 16 + t16, last_tok)], p.max_slot);
     };
     auto load_tile = [&](KvTile<D>& t, int s0, int s1) {
 #pragma unroll
@@ -701,6 +702,7 @@ int launch_splitkv(const SplitKvArgs& a, hipStream_t stream) {
   p.n_q = (int32_t)a.n_q;
   p.n_kv = (int32_t)a.n_kv;
   p.group = (int32_t)group;
+  p.max_slot = (uint32_t)(a.num_slots > 0 ? a.num_slots - 1 : 0);
   p.nwh = nwh;
   p.head_groups = (int32_t)(a.n_kv / nwh);
   p.n_seg = a.n_seg;
