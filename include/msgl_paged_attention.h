@@ -276,6 +276,9 @@ MSGL_API int msgl_gdn_state_inplace(const void* q, const void* k, const void* v,
  *                            4 waves x 64 rows; 2: head_dim 256 through split-K in query chunks
  *   MSGL_TUNE_SPLITKV_WAVES  most waves (adjacent kv heads) per split-K workgroup: 1, 2, 4, 8
  *                            (0 restores the default, 4)
+ *   MSGL_TUNE_SPLITKV_BOUNDARY tokens' worth of time a split-K workgroup is charged for starting
+ *                            on another request inside its segment (0: default from the shape,
+ *                            negative: none)
  *   MSGL_TUNE_GDN_ROWS       state rows per 16-lane group of the gdn_state kernel: 1, 2, 4
  *                            (0: chosen from the problem size)
  *   MSGL_TUNE_PREFILL_KEY_SPLITS  workgroups that share the keys of one query block of the MFMA
@@ -288,6 +291,7 @@ MSGL_API int msgl_gdn_state_inplace(const void* q, const void* k, const void* v,
 #define MSGL_TUNE_SPLITKV_WAVES 4
 #define MSGL_TUNE_GDN_ROWS 5
 #define MSGL_TUNE_PREFILL_KEY_SPLITS 6
+#define MSGL_TUNE_SPLITKV_BOUNDARY 7
 MSGL_API int msgl_set_tuning(int32_t knob, int64_t value);
 
 #ifdef __cplusplus

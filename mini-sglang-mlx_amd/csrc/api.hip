@@ -86,6 +86,10 @@ int msgl_set_tuning(int32_t knob, int64_t value) {
     msgl::splitkv_set_max_waves((int)value);
     return MSGL_OK;
   }
+  if (knob == MSGL_TUNE_SPLITKV_BOUNDARY) {
+    msgl::splitkv_set_boundary((int)value);
+    return MSGL_OK;
+  }
   if (knob == MSGL_TUNE_GDN_ROWS) {
     msgl::gdn_set_rows((int)value);
     return MSGL_OK;

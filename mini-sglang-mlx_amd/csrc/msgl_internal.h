@@ -46,6 +46,8 @@ constexpr int kSplitKvMinSegment = 128;
 // one resident round of workgroups for this shape, capped so segments keep min_seg tokens
 int splitkv_default_segments(int64_t total_kv, int64_t n_kv, int64_t head_dim, int64_t cols,
                              int32_t min_seg);
+// benchmarking switch: stream positions charged per request boundary (0: default, negative: none)
+void splitkv_set_boundary(int v);
 size_t splitkv_workspace_bytes(int64_t batch, int64_t n_q, int64_t n_kv, int64_t head_dim,
                                int64_t max_len_extend, int32_t n_seg);
 int launch_splitkv(const SplitKvArgs& a, hipStream_t stream);

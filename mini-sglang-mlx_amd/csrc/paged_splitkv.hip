@@ -55,7 +55,7 @@ struct SplitKvParams {
   const int32_t* qo_indptr;
   const int32_t* prefix_lens;
   uint16_t* out;
-  float* part_o;        // [n_seg + batch][n_kv][cols][D]
+  float* part_o;        // [n_seg + batch][n_kv][D / 8][cols][8]: see partial_offset()
   float* part_lse;      // [n_seg + batch][n_kv][cols]
   int32_t* req_items;   // [batch][2] first segment holding the request, number of segments sharing it
   int64_t k_stride0, v_stride0;
@@ -63,6 +63,7 @@ struct SplitKvParams {
   int32_t nwh;          // kv heads per workgroup
   int32_t head_groups;  // n_kv / nwh
   int32_t n_seg, min_seg, cols, max_len_extend;
+  int32_t boundary;  // stream positions a request boundary is charged with (see stream_length)
   int32_t q_begin, q_cap;  // first query of every request in this launch; cap on a request's queries
   int32_t f16;             // elements are IEEE half instead of bf16
   int32_t is_cross, window;
@@ -107,13 +108,39 @@ __device__ __forceinline__ ReqInfo request_info(const SplitKvParams& p, int b) {
   return r;
 }
 
+// Where dim `dim` of column `col` of the partial of (item, kv head) number `block` lives.  Blocks
+// of 8 dims are the outer index and columns the inner one: in the attention kernel's accumulator
+// layout the 16 lanes of a row group hold the same 8 dims of 16 consecutive columns, so one store
+// instruction writes 32 contiguous bytes per lane and 512 contiguous bytes per row group.  (With
+// the column as the outer index every lane of a store wrote 16 bytes of a different 512-byte row:
+// 64 partial cache lines per instruction, and the partial stores of a share cost as much as
+// several microseconds of streaming.)
+__device__ __forceinline__ int64_t partial_offset(int64_t block, int cols, int col, int dim, int D) {
+  return (block * cols * (int64_t)D) + ((int64_t)(dim >> 3) * cols + col) * 8 + (dim & 7);
+}
+
+// A request with visible keys takes their number of positions in the stream plus `boundary`
+// positions without tokens behind them.  Starting on the next request costs a workgroup a fixed
+// time (its geometry, Q rows, slot ids and first tiles are three dependent memory round trips, and
+// the load pipeline drains and refills): measured 8-9 us, the time of about a hundred tokens, and the
+// kernel ends when its slowest workgroup does.  Charging the boundary to the segment that crosses it
+// gives that workgroup fewer tokens; a segment that ends or starts inside the empty positions just
+// has less to do or starts at the next request.
+__device__ __forceinline__ int stream_length(const SplitKvParams& p, int visible) {
+  return visible > 0 ? visible + p.boundary : 0;
+}
+
+// Segments are a multiple of 64 positions long, one trip of the tile loop.  (Multiples of 16 or 32
+// fill the last few segments that rounding up to 64 leaves without work, but give every share a
+// partly filled trip: measured 0.5-1 % slower on the decode and verify shapes.)
 __device__ __forceinline__ int segment_length(int total, int n_seg, int min_seg) {
   const int even = ((total + n_seg - 1) / n_seg + 63) / 64 * 64;
   return max(even, min_seg);
 }
 
-// Wave-cooperative: length of the visible token stream, and the request that holds stream
-// position `seg * seg_len` together with the stream position of that request's first key.
+// Wave-cooperative: length of the stream, and the request that holds stream position
+// `seg * seg_len` (its keys or the empty positions behind them) together with the stream position
+// of that request's first key.
 // Returns false when the segment starts beyond the stream.  All lanes must call.
 __device__ __forceinline__ bool locate_segment(const SplitKvParams& p, int seg, int* seg_len,
                                                int* total_out, int* req, int* req_vstart) {
@@ -124,7 +151,7 @@ __device__ __forceinline__ bool locate_segment(const SplitKvParams& p, int seg, 
     n = 0;
     if (b < p.batch) {
       const ReqInfo r = request_info(p, b);
-      n = r.hi - r.lo;
+      n = stream_length(p, r.hi - r.lo);
     }
     incl = wave_inclusive_scan(n);
     total += __shfl(incl, kWave - 1, kWave);
@@ -141,7 +168,7 @@ __device__ __forceinline__ bool locate_segment(const SplitKvParams& p, int seg, 
       n = 0;
       if (b < p.batch) {
         const ReqInfo r = request_info(p, b);
-        n = r.hi - r.lo;
+        n = stream_length(p, r.hi - r.lo);
       }
       incl = wave_inclusive_scan(n);
     }
@@ -200,10 +227,12 @@ __global__ __launch_bounds__(64 * NW, ((D == 128 && NCT == 1) ? 2 : 1)) void spl
     else return (uint64_t)((uint32_t)slot_id * row_bytes);
   };
 
-  while (vpos < seg_end) {
+  while (vpos < seg_end && cur_b < p.batch) {
     const ReqInfo r = request_info(p, cur_b);
     const int vlen = r.hi - r.lo;
-    if (vlen == 0) {
+    if (vpos >= vs + vlen) {  // no keys, or past them in the empty positions: on to the next request
+      vs += stream_length(p, vlen);
+      vpos = max(vpos, vs);
       ++cur_b;
       continue;
     }
@@ -421,8 +450,7 @@ __global__ __launch_bounds__(64 * NW, ((D == 128 && NCT == 1) ? 2 : 1)) void spl
             st_global_b128(orow + hf * 128 + (4 * g + i) * 8, w);
           }
       } else {
-        const int64_t prow = ((int64_t)(seg + cur_b) * p.n_kv + kvh) * p.cols + col;
-        float* po = p.part_o + prow * D;
+        const int64_t block = (int64_t)(seg + cur_b) * p.n_kv + kvh;
 #pragma unroll
         for (int hf = 0; hf < VH; ++hf)
 #pragma unroll
@@ -433,17 +461,15 @@ __global__ __launch_bounds__(64 * NW, ((D == 128 && NCT == 1) ? 2 : 1)) void spl
               w0[n] = oacc[ct][hf][n][i] * inv;
               w1[n] = oacc[ct][hf][4 + n][i] * inv;
             }
-            float* dst = po + hf * 128 + (4 * g + i) * 8;
+            float* dst = p.part_o + partial_offset(block, p.cols, col, hf * 128 + (4 * g + i) * 8, D);
             *reinterpret_cast<f32x4_t*>(dst) = w0;
             *reinterpret_cast<f32x4_t*>(dst + 4) = w1;
           }
-        if (g == 0) p.part_lse[prow] = (l > 0.f) ? m_run[ct] + __log2f(l) : kNegInf;
+        if (g == 0) p.part_lse[block * p.cols + col] = (l > 0.f) ? m_run[ct] + __log2f(l) : kNegInf;
       }
     }
 
-    vpos += t_end - t_begin;
-    vs += vlen;
-    ++cur_b;
+    vpos += t_end - t_begin;  // the request's end, or the segment's: the loop head sorts it out
   }
 }
 
@@ -472,14 +498,15 @@ __global__ __launch_bounds__(64) void splitkv_merge_kernel(SplitKvParams p) {
   if (n_items == 1) return;  // written by the attention kernel itself
   const int kvh = hq / p.group;
   const int col = qi * p.group + (hq - kvh * p.group);
-  const int64_t stride = (int64_t)p.n_kv * p.cols;
-  const int64_t row0 = ((int64_t)(s_first + b) * p.n_kv + kvh) * p.cols + col;
+  const int64_t stride = (int64_t)p.n_kv * p.cols;                               // rows per item
+  const int64_t row0 = ((int64_t)(s_first + b) * p.n_kv + kvh) * p.cols + col;  // LSE of item 0
+  const int64_t block0 = (int64_t)(s_first + b) * p.n_kv + kvh;                 // partial of item 0
 
   constexpr int kAhead = 4;  // partial rows requested before their weights are known
   float v[kAhead][PER];
 #pragma unroll
   for (int u = 0; u < kAhead; ++u) {
-    const float* src = p.part_o + (row0 + min(u, n_items - 1) * stride) * D + lane * PER;
+    const float* src = p.part_o + partial_offset(block0 + (int64_t)min(u, n_items - 1) * p.n_kv, p.cols, col, lane * PER, D);
 #pragma unroll
     for (int e = 0; e < PER; ++e) v[u][e] = src[e];
   }
@@ -509,7 +536,7 @@ __global__ __launch_bounds__(64) void splitkv_merge_kernel(SplitKvParams p) {
     for (int it = kAhead; it < n_items; ++it) {
       const int64_t row = row0 + it * stride;
       const float wu = fast_exp2(p.part_lse[row] - mx);
-      const float* src = p.part_o + row * D + lane * PER;
+      const float* src = p.part_o + partial_offset(block0 + (int64_t)it * p.n_kv, p.cols, col, lane * PER, D);
 #pragma unroll
       for (int e = 0; e < PER; ++e) acc[e] += wu * src[e];
       wsum += wu;
@@ -631,6 +658,21 @@ int splitkv_scratch(void** ptr, size_t* bytes) {
 
 void splitkv_set_max_waves(int v) { t_max_waves = v > 0 ? v : 4; }  // 0 restores the default
 
+// benchmarking switch, one value per host thread: stream positions charged per request boundary
+// (0: chosen from the shape, below; negative: none)
+static thread_local int t_boundary = 0;
+void splitkv_set_boundary(int v) { t_boundary = v; }
+// A boundary costs a workgroup about 8 us (measured on the benchmark shapes, one and eight
+// queries per request); in that time it would stream 8 us x (what the chip reads per us) /
+// (workgroups x bytes of one token's K and V rows for the workgroup's kv heads) tokens.
+static int boundary_tokens(int64_t n_wgs, int nwh, int64_t head_dim) {
+  if (t_boundary != 0) return t_boundary > 0 ? (t_boundary < 4096 ? t_boundary : 4096) : 0;
+  const double bytes_per_token = (double)nwh * 2.0 * (double)head_dim * 2.0;
+  const double tokens = 8.0 * 6.2e6 / ((double)(n_wgs > 0 ? n_wgs : 1) * bytes_per_token);
+  const int64_t t = ((int64_t)tokens + 8) / 16 * 16;
+  return (int)(t < 0 ? 0 : (t > 1024 ? 1024 : t));
+}
+
 // kv heads per workgroup for this shape: up to 4, halved when a second wave per head is
 // needed for the columns (a workgroup of the wide variants holds at most 4 waves: they
 // need more than 256 VGPRs, one wave per SIMD)
@@ -706,6 +748,7 @@ int launch_splitkv(const SplitKvArgs& a, hipStream_t stream) {
   p.nwh = nwh;
   p.head_groups = (int32_t)(a.n_kv / nwh);
   p.n_seg = a.n_seg;
+  p.boundary = boundary_tokens((int64_t)a.n_seg * (a.n_kv / nwh), nwh, a.head_dim);
   p.min_seg = a.min_seg;
   p.max_len_extend = a.max_len_extend;
   p.f16 = a.f16;

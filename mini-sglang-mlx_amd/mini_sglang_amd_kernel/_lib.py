@@ -86,6 +86,7 @@ TUNE_PREFILL_VARIANT = 3
 TUNE_SPLITKV_WAVES = 4
 TUNE_GDN_ROWS = 5
 TUNE_PREFILL_KEY_SPLITS = 6
+TUNE_SPLITKV_BOUNDARY = 7
 
 _lib = None
 
