@@ -114,3 +114,47 @@ def test_cfg5_speculative_verify_full_oracle(gpu, variant):
     print("cfg5 oracle", flush=True)
     want, _ = run_oracle(wl, precision="f32")
     assert_close_bf16(got, want, f"cfg5 {variant}")
+
+
+def _uniform_attention_expected(g):
+    """With q = 0 every visible key weighs the same, so a row's output is the plain mean of the
+    V rows it may see: sums in float64 (torch on the GPU as the adding machine), no oracle."""
+    group = g.n_q // g.n_kv
+    ip = g.kv_indptr.tolist()
+    window, cross = g.sliding_window_size, g.is_cross_attention
+    outs = []
+    for b in range(g.batch):
+        rows = g.v_cache[g.kv_indices[ip[b]:ip[b + 1]].long()].double()  # (kv_len, n_kv, d)
+        kv_len = rows.shape[0]
+        if g.kind == "decode":
+            mean = rows.sum(0, keepdim=True) / kv_len
+        else:
+            ext = g.extend_lens[b]
+            before = torch.cat([torch.zeros_like(rows[:1]), rows.cumsum(0)])  # sum of keys < t
+            pos = (kv_len - ext) + torch.arange(ext, device=rows.device)
+            hi = torch.full_like(pos, kv_len - 1) if cross else pos
+            lo = torch.clamp(pos - window + 1, min=0) if window > 0 else torch.zeros_like(pos)
+            mean = (before[hi + 1] - before[lo]) / (hi + 1 - lo).double()[:, None, None]
+        outs.append(mean.repeat_interleave(group, dim=1))
+        del rows
+    return torch.cat(outs)
+
+
+@pytest.mark.parametrize("cfg,variant", [(2, ""), (3, ""), (4, ""), (5, ""), (5, "window")])
+def test_uniform_attention_closed_form_every_row_full_size(gpu, cfg, variant):
+    """Full size, every request, every row and head, against a closed form: q = 0 makes the
+    weights exactly 1 / (visible keys), so a dropped, doubled or wrongly gathered key, a
+    wrong causal limit or window floor, or a mis-merged segment moves the result by about
+    |v| / keys, which the bound below (bf16 rounding of the result plus 2e-5) does not cover
+    for a v of ordinary size."""
+    print(f"cfg{cfg} {variant} uniform attention: build", flush=True)
+    wl = config_workload(cfg, variant=variant, **({"pool_device": gpu} if cfg == 4 else {}))
+    wl.q.zero_()
+    got, g = run_gpu(wl, gpu)
+    print(f"cfg{cfg} {variant} uniform attention: closed form", flush=True)
+    want = _uniform_attention_expected(g)
+    diff = (got.to(gpu).double() - want).abs()
+    bound = want.abs() * 2.0 ** -8 + 2e-5
+    worst = float((diff - bound).max())
+    assert worst <= 0.0, (f"cfg{cfg} {variant}: a row is {worst:.3e} beyond its bound; "
+                          f"max-abs diff {float(diff.max()):.3e}")
