@@ -158,3 +158,73 @@ def test_uniform_attention_closed_form_every_row_full_size(gpu, cfg, variant):
     worst = float((diff - bound).max())
     assert worst <= 0.0, (f"cfg{cfg} {variant}: a row is {worst:.3e} beyond its bound; "
                           f"max-abs diff {float(diff.max()):.3e}")
+
+
+def _needle_queries(g, gap_nats=28.0):
+    """A query per (row, q head) that points at ONE visible key of its own: q = c k* / |k*|^2,
+    with c large enough that the softmax weight of every other key is below e^-gap.  Targets
+    cycle through the last visible key (the causal limit / the diagonal tile), the first visible
+    key (position 0 or the window floor) and one in between.  Returns (q, expected output):
+    the expected row is the target's V row, bit for bit."""
+    group = g.n_q // g.n_kv
+    ip = g.kv_indptr.tolist()
+    window, cross = g.sliding_window_size, g.is_cross_attention
+    dev = g.k_cache.device
+    head = torch.arange(g.n_q, device=dev)
+    qs, wants = [], []
+    row0 = 0
+    for b in range(g.batch):
+        idx = g.kv_indices[ip[b]:ip[b + 1]].long()
+        kv_len, ext = idx.numel(), g.extend_lens[b]
+        pos = (kv_len - ext) + torch.arange(ext, device=dev)
+        hi = torch.full_like(pos, kv_len - 1) if (cross or g.kind == "decode") else pos
+        lo = torch.clamp(pos - window + 1, min=0) if window > 0 else torch.zeros_like(pos)
+        pick = (row0 + torch.arange(ext, device=dev))[:, None] + head[None, :]  # (ext, n_q)
+        mid = lo[:, None] + (pick * 7919) % (hi - lo + 1)[:, None]
+        target = torch.where(pick % 3 == 0, hi[:, None], torch.where(pick % 3 == 1, lo[:, None], mid))
+        slot = idx[target]                                         # (ext, n_q)
+        kvh = (head // group)[None, :].expand_as(slot)
+        k_star = g.k_cache[slot, kvh].double()                     # (ext, n_q, d)
+        norm2 = (k_star * k_star).sum(-1)                          # (ext, n_q)
+        u = k_star / norm2[..., None]
+        # other keys' logits relative to the target's: k_j . k* / |k*|^2, largest over the request
+        # (keys the row cannot see included: that only makes c larger than needed)
+        k_heads = g.k_cache[idx][:, head // group].float()         # (kv_len, n_q, d)
+        ratio = torch.einsum("thd,ehd->eht", k_heads, u.float())   # (ext, n_q, kv_len)
+        ratio.scatter_(2, target[..., None], float("-inf"))
+        worst = ratio.max(dim=2).values.double().clamp(min=0.0)
+        assert float(worst.max()) < 0.9, "another key is nearly parallel to a target"
+        c = gap_nats / (g.sm_scale * (1.0 - worst))
+        del k_heads, ratio
+        qs.append((u * c[..., None]).to(torch.bfloat16))
+        wants.append(g.v_cache[slot, kvh])
+        row0 += ext
+    return torch.cat(qs), torch.cat(wants)
+
+
+@pytest.mark.parametrize("cfg,variant", [(2, ""), (3, ""), (4, ""), (5, ""), (5, "window")])
+def test_needle_queries_return_their_key_every_row_full_size(gpu, cfg, variant):
+    """Full size, every request, row and head, no oracle: each query points at one visible key
+    (its last, its first, or one in between), every other key's weight is below e^-28, so the
+    row must be that key's V row.  Pins what the uniform-attention check leaves open: the QK
+    product, K and V gathered by the same slot id, and the score path at the mask edges (a
+    target wrongly masked, or a key beyond the edge wrongly seen, changes the whole row)."""
+    from mini_sglang_amd_kernel import store_kv_cache
+
+    print(f"cfg{cfg} {variant} needle queries: build", flush=True)
+    wl = config_workload(cfg, variant=variant, **({"pool_device": gpu} if cfg == 4 else {}))
+    g = wl.to(gpu)
+    if g.out_loc is not None:
+        store_kv_cache(g.k_cache, g.v_cache, g.out_loc, g.new_k, g.new_v)
+    q, want = _needle_queries(g)
+    g.q = q.reshape(g.q.shape)
+    print(f"cfg{cfg} {variant} needle queries: run", flush=True)
+    got, _ = run_gpu(g, gpu, store=False)
+    got = got.to(gpu).reshape(want.shape)
+    exact = (got.view(torch.int16) == want.view(torch.int16)).all(dim=-1)
+    diff = (got.double() - want.double()).abs()
+    bound = want.double().abs() * 2.0 ** -8 + 1e-6
+    assert bool((diff <= bound).all()), (
+        f"cfg{cfg} {variant}: {int((~(diff <= bound).all(dim=-1)).sum())} rows are not their "
+        f"target's V row; max-abs diff {float(diff.max()):.3e}")
+    assert float(exact.double().mean()) > 0.99, "fewer than 99 % of the rows are bit-exact copies"
