@@ -116,6 +116,15 @@ def test_cfg5_speculative_verify_full_oracle(gpu, variant):
     assert_close_bf16(got, want, f"cfg5 {variant}")
 
 
+_FULL_SIZE_SHAPES = [(2, ""), (3, ""), (3, "head_dim_256"), (4, ""), (5, ""), (5, "window")]
+
+
+def _full_size_workload(cfg, variant, gpu):
+    if variant == "head_dim_256":
+        return config_workload(cfg, head_dim=256)
+    return config_workload(cfg, variant=variant, **({"pool_device": gpu} if cfg == 4 else {}))
+
+
 def _uniform_attention_expected(g):
     """With q = 0 every visible key weighs the same, so a row's output is the plain mean of the
     V rows it may see: sums in float64 (torch on the GPU as the adding machine), no oracle."""
@@ -140,7 +149,7 @@ def _uniform_attention_expected(g):
     return torch.cat(outs)
 
 
-@pytest.mark.parametrize("cfg,variant", [(2, ""), (3, ""), (4, ""), (5, ""), (5, "window")])
+@pytest.mark.parametrize("cfg,variant", _FULL_SIZE_SHAPES)
 def test_uniform_attention_closed_form_every_row_full_size(gpu, cfg, variant):
     """Full size, every request, every row and head, against a closed form: q = 0 makes the
     weights exactly 1 / (visible keys), so a dropped, doubled or wrongly gathered key, a
@@ -148,7 +157,7 @@ def test_uniform_attention_closed_form_every_row_full_size(gpu, cfg, variant):
     |v| / keys, which the bound below (bf16 rounding of the result plus 2e-5) does not cover
     for a v of ordinary size."""
     print(f"cfg{cfg} {variant} uniform attention: build", flush=True)
-    wl = config_workload(cfg, variant=variant, **({"pool_device": gpu} if cfg == 4 else {}))
+    wl = _full_size_workload(cfg, variant, gpu)
     wl.q.zero_()
     got, g = run_gpu(wl, gpu)
     print(f"cfg{cfg} {variant} uniform attention: closed form", flush=True)
@@ -202,7 +211,7 @@ def _needle_queries(g, gap_nats=28.0):
     return torch.cat(qs), torch.cat(wants)
 
 
-@pytest.mark.parametrize("cfg,variant", [(2, ""), (3, ""), (4, ""), (5, ""), (5, "window")])
+@pytest.mark.parametrize("cfg,variant", _FULL_SIZE_SHAPES)
 def test_needle_queries_return_their_key_every_row_full_size(gpu, cfg, variant):
     """Full size, every request, row and head, no oracle: each query points at one visible key
     (its last, its first, or one in between), every other key's weight is below e^-28, so the
@@ -212,7 +221,7 @@ def test_needle_queries_return_their_key_every_row_full_size(gpu, cfg, variant):
     from mini_sglang_amd_kernel import store_kv_cache
 
     print(f"cfg{cfg} {variant} needle queries: build", flush=True)
-    wl = config_workload(cfg, variant=variant, **({"pool_device": gpu} if cfg == 4 else {}))
+    wl = _full_size_workload(cfg, variant, gpu)
     g = wl.to(gpu)
     if g.out_loc is not None:
         store_kv_cache(g.k_cache, g.v_cache, g.out_loc, g.new_k, g.new_v)
