@@ -39,6 +39,7 @@
 // Algorithmic HBM bytes per visible token and kv head: 2 * D * 2 (one K row + one V row)
 // plus 4 bytes of kv_indices per token.
 #include <atomic>
+#include <type_traits>
 
 #include "msgl_device.h"
 #include "msgl_internal.h"
@@ -473,26 +474,39 @@ __global__ __launch_bounds__(64 * NW, ((D == 128 && NCT == 1) ? 2 : 1)) void spl
   }
 }
 
-// One wave per (request, query, q head): merge the partials of the segments that share
-// the request, by base-2 LSE.  Requests without visible keys get zeros; requests that sat
-// inside one segment were written by the attention kernel itself.
-template <int D, bool F16>
-__global__ __launch_bounds__(64) void splitkv_merge_kernel(SplitKvParams p) {
+// One workgroup of NW waves per (request, query, q head): merge the partials of the segments
+// that share the request, by base-2 LSE.  Requests without visible keys get zeros; requests
+// that sat inside one segment were written by the attention kernel itself.
+// Up to kMergeSmall items (a request cut a few times: the usual case) one wave reads whole rows
+// and nothing crosses lanes.  Beyond that a partial row is taken as D / 8 chunks of 8 floats,
+// one chunk per lane, so a wave holds 64 / (D / 8) rows side by side and a workgroup
+// NG = NW * that many; each of these lane groups takes every NG-th item, one in the first trip
+// and kMergeUnroll per trip after it, with all their loads in flight together.  A request cut
+// into a hundred segments (one long request alone on the chip) thus needs three or four memory
+// round trips where a loop over its items needs a hundred.
+constexpr int kMergeUnroll = 3;
+constexpr int kMergeSmall = 8;
+template <int D, bool F16, int NW>
+__global__ __launch_bounds__(64 * NW) void splitkv_merge_kernel(SplitKvParams p) {
+  constexpr int LPI = D / 8;          // lanes per item
+  constexpr int GPW = kWave / LPI;    // items side by side in a wave
+  constexpr int NG = GPW * NW;        // ... and in the workgroup
+  constexpr int U = kMergeUnroll;
   const int b = blockIdx.x / p.max_len_extend;
   const int qi = blockIdx.x - b * p.max_len_extend;
   const int hq = blockIdx.y;
   const int lane = lane_id();
-  // two memory round trips in all: the request's geometry and the place of its partials,
-  // then every LSE and the first partial rows together
+  const int wave = threadIdx.x >> 6;
+  const int grp = wave * GPW + lane / LPI;
+  const int dl = lane % LPI;  // this lane's chunk: dims dl * 8 .. dl * 8 + 7
+  // every exit below, and the choice between the two ways, is the same for the whole workgroup
   const int s_first = p.req_items[2 * b];
   const int n_items = p.req_items[2 * b + 1];
   const ReqInfo r = request_info(p, b);
   if (qi >= r.q_len) return;
-  constexpr int PER = D / kWave;  // consecutive floats per lane
-  uint16_t* orow = p.out + ((int64_t)(r.q_start + qi) * p.n_q + hq) * D + lane * PER;
+  uint16_t* orow = p.out + ((int64_t)(r.q_start + qi) * p.n_q + hq) * D + dl * 8;
   if (r.hi - r.lo == 0) {  // no visible key: nobody wrote req_items, the row is zero
-#pragma unroll
-    for (int e = 0; e < PER; ++e) orow[e] = 0;
+    if (threadIdx.x < LPI) st_global_b128(orow, u32x4_t{0u, 0u, 0u, 0u});
     return;
   }
   if (n_items == 1) return;  // written by the attention kernel itself
@@ -502,50 +516,130 @@ __global__ __launch_bounds__(64) void splitkv_merge_kernel(SplitKvParams p) {
   const int64_t row0 = ((int64_t)(s_first + b) * p.n_kv + kvh) * p.cols + col;  // LSE of item 0
   const int64_t block0 = (int64_t)(s_first + b) * p.n_kv + kvh;                 // partial of item 0
 
-  constexpr int kAhead = 4;  // partial rows requested before their weights are known
-  float v[kAhead][PER];
+  if (n_items <= kMergeSmall) {
+    // one wave, a whole row per load, every lane reads the few LSEs itself: one memory round
+    // trip after the geometry's
+    if (wave > 0) return;
+    constexpr int PER = D / kWave;  // consecutive floats per lane
+    float ls[kMergeSmall], v[kMergeSmall][PER];
 #pragma unroll
-  for (int u = 0; u < kAhead; ++u) {
-    const float* src = p.part_o + partial_offset(block0 + (int64_t)min(u, n_items - 1) * p.n_kv, p.cols, col, lane * PER, D);
+    for (int u = 0; u < kMergeSmall; ++u) {
+      ls[u] = kNegInf;
 #pragma unroll
-    for (int e = 0; e < PER; ++e) v[u][e] = src[e];
-  }
-  float my_lse = kNegInf;  // lane i holds the LSE of item i (+ 64, + 128, ... folded by max)
-  float mx = kNegInf;
-  for (int it = lane; it < n_items; it += kWave) {
-    const float x = p.part_lse[row0 + it * stride];
-    if (it < kWave) my_lse = x;
-    mx = fmaxf(mx, x);
-  }
-#pragma unroll
-  for (int off = 1; off < kWave; off <<= 1) mx = fmaxf(mx, __shfl_xor(mx, off, kWave));
-  float acc[PER];
-#pragma unroll
-  for (int e = 0; e < PER; ++e) acc[e] = 0.f;
-  float wsum = 0.f;
-  if (mx > kNegInf) {
-#pragma unroll
-    for (int u = 0; u < kAhead; ++u) {
+      for (int e = 0; e < PER; ++e) v[u][e] = 0.f;
       if (u < n_items) {
-        const float wu = fast_exp2(__shfl(my_lse, u, kWave) - mx);
+        ls[u] = p.part_lse[row0 + u * stride];
+        const float* src = p.part_o + partial_offset(block0 + (int64_t)u * p.n_kv, p.cols, col, lane * PER, D);
+#pragma unroll
+        for (int e = 0; e < PER; ++e) v[u][e] = src[e];
+      }
+    }
+    float mx = ls[0];
+#pragma unroll
+    for (int u = 1; u < kMergeSmall; ++u) mx = fmaxf(mx, ls[u]);
+    float acc[PER];
+#pragma unroll
+    for (int e = 0; e < PER; ++e) acc[e] = 0.f;
+    float wsum = 0.f;
+    if (mx > kNegInf) {
+#pragma unroll
+      for (int u = 0; u < kMergeSmall; ++u) {
+        const float wu = fast_exp2(ls[u] - mx);  // 0 for an item that is not there
 #pragma unroll
         for (int e = 0; e < PER; ++e) acc[e] += wu * v[u][e];
         wsum += wu;
       }
     }
-    for (int it = kAhead; it < n_items; ++it) {
-      const int64_t row = row0 + it * stride;
-      const float wu = fast_exp2(p.part_lse[row] - mx);
-      const float* src = p.part_o + partial_offset(block0 + (int64_t)it * p.n_kv, p.cols, col, lane * PER, D);
+    const float inv = (wsum > 0.f) ? 1.0f / wsum : 0.f;
+    uint16_t* dst = p.out + ((int64_t)(r.q_start + qi) * p.n_q + hq) * D + lane * PER;
 #pragma unroll
-      for (int e = 0; e < PER; ++e) acc[e] += wu * src[e];
+    for (int e = 0; e < PER; e += 2)
+      *reinterpret_cast<uint32_t*>(dst + e) = pack_16x2<F16>(acc[e] * inv, acc[e + 1] * inv);
+    return;
+  }
+
+  float acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+  float wsum = 0.f;
+  float lse[U];
+  f32x4_t va[U][2];
+  // items base, base + NG, ... (`n` of them); lanes past the last item load nothing and
+  // contribute weight 0 to a row of zeros
+  auto fetch = [&](int base, auto n) {
+#pragma unroll
+    for (int u = 0; u < decltype(n)::value; ++u) {
+      const int it = base + u * NG;
+      lse[u] = kNegInf;
+      va[u][0] = va[u][1] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      if (it < n_items) {
+        lse[u] = p.part_lse[row0 + it * stride];
+        const float* src = p.part_o + partial_offset(block0 + (int64_t)it * p.n_kv, p.cols, col, dl * 8, D);
+        va[u][0] = *reinterpret_cast<const f32x4_t*>(src);
+        va[u][1] = *reinterpret_cast<const f32x4_t*>(src + 4);
+      }
+    }
+  };
+  auto consume = [&](float mx, auto n) {
+#pragma unroll
+    for (int u = 0; u < decltype(n)::value; ++u) {
+      const float wu = fast_exp2(lse[u] - mx);  // 0 for an item that is not there
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        acc[e] += wu * va[u][0][e];
+        acc[4 + e] += wu * va[u][1][e];
+      }
       wsum += wu;
     }
-  }
-  const float inv = (wsum > 0.f) ? 1.0f / wsum : 0.f;
+  };
+  using One = std::integral_constant<int, 1>;
+  using Trip = std::integral_constant<int, U>;
+  // Two memory round trips for up to NG items: geometry and place of the partials above, then
+  // every LSE (for the maximum) and one row per lane group together.  The rest in trips of
+  // NG * U items.
+  fetch(grp, One{});
+  float mx = kNegInf;
+  for (int it = lane; it < n_items; it += kWave) mx = fmaxf(mx, p.part_lse[row0 + it * stride]);
 #pragma unroll
-  for (int e = 0; e < PER; e += 2)
-    *reinterpret_cast<uint32_t*>(orow + e) = pack_16x2<F16>(acc[e] * inv, acc[e + 1] * inv);
+  for (int off = 1; off < kWave; off <<= 1) mx = fmaxf(mx, __shfl_xor(mx, off, kWave));
+  if (mx > kNegInf) {
+    consume(mx, One{});
+    for (int base = grp + NG; base < n_items; base += NG * U) {
+      fetch(base, Trip{});
+      consume(mx, Trip{});
+    }
+  }
+  // fold the lane groups of a wave, then the waves
+#pragma unroll
+  for (int off = LPI; off < kWave; off <<= 1) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] += __shfl_xor(acc[e], off, kWave);
+    wsum += __shfl_xor(wsum, off, kWave);
+  }
+  if constexpr (NW > 1) {
+    __shared__ float fold[NW - 1][LPI][9];
+    if (wave > 0 && lane < LPI) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) fold[wave - 1][lane][e] = acc[e];
+      fold[wave - 1][lane][8] = wsum;
+    }
+    __syncthreads();
+    if (wave > 0) return;
+    if (lane < LPI) {
+#pragma unroll
+      for (int w = 0; w < NW - 1; ++w) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] += fold[w][lane][e];
+        wsum += fold[w][lane][8];
+      }
+    }
+  }
+  if (lane >= LPI) return;
+  const float inv = (wsum > 0.f) ? 1.0f / wsum : 0.f;
+  u32x4_t w;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) w[e] = pack_16x2<F16>(acc[2 * e] * inv, acc[2 * e + 1] * inv);
+  st_global_b128(orow, w);
 }
 
 int nct_for(int64_t cols) { return (int)((cols + 15) / 16); }
@@ -603,8 +697,17 @@ int launch_dn(const SplitKvParams& p, int waves, hipStream_t stream) {
   int rc = check_launch();
   if (rc != MSGL_OK) return rc;
   const dim3 mgrid((unsigned)(p.batch * p.max_len_extend), (unsigned)p.n_q);
-  if (p.f16) hipLaunchKernelGGL((splitkv_merge_kernel<D, true>), mgrid, dim3(64), 0, stream, p);
-  else hipLaunchKernelGGL((splitkv_merge_kernel<D, false>), mgrid, dim3(64), 0, stream, p);
+  // four waves per row when a request can be cut into more items than one wave takes in a trip
+  // and the rows are few enough that the extra waves cost nothing
+  constexpr int kItemsPerTrip = kWave / (D / 8) * (1 + kMergeUnroll);
+  const bool wide_merge = p.n_seg > kItemsPerTrip && (int64_t)mgrid.x * mgrid.y <= 1024;
+  if (wide_merge) {
+    if (p.f16) hipLaunchKernelGGL((splitkv_merge_kernel<D, true, 4>), mgrid, dim3(256), 0, stream, p);
+    else hipLaunchKernelGGL((splitkv_merge_kernel<D, false, 4>), mgrid, dim3(256), 0, stream, p);
+  } else {
+    if (p.f16) hipLaunchKernelGGL((splitkv_merge_kernel<D, true, 1>), mgrid, dim3(64), 0, stream, p);
+    else hipLaunchKernelGGL((splitkv_merge_kernel<D, false, 1>), mgrid, dim3(64), 0, stream, p);
+  }
   return check_launch();
 }
 

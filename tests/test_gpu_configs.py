@@ -237,3 +237,32 @@ def test_needle_queries_return_their_key_every_row_full_size(gpu, cfg, variant):
         f"cfg{cfg} {variant}: {int((~(diff <= bound).all(dim=-1)).sum())} rows are not their "
         f"target's V row; max-abs diff {float(diff.max()):.3e}")
     assert float(exact.double().mean()) > 0.99, "fewer than 99 % of the rows are bit-exact copies"
+
+
+@pytest.mark.parametrize("head_dim", [128, 256])
+@pytest.mark.parametrize("lens,ext", [([40000], 1), ([70000, 300, 5000], 1), ([30000], 8),
+                                      ([20000, 900], 3)])
+def test_few_long_requests_merge_of_many_partials(gpu, lens, ext, head_dim):
+    """One long request alone (or beside short ones) is cut into as many segments as the chip
+    has workgroups, so the merge sees up to a hundred partials per row: both closed forms
+    (uniform weights, needle queries), every row and head, decode and short query blocks."""
+    from mini_sglang_amd.workloads import build_workload
+
+    kind = "decode" if ext == 1 else "prefill"
+    wl = build_workload(f"long_{lens}_{ext}", kind, seed=7, n_q=16, n_kv=4, head_dim=head_dim,
+                        kv_lens=lens, extend_lens=[ext] * len(lens), pool_device=gpu)
+    g = wl.to(gpu)
+    q_rand = g.q.clone()
+    g.q = torch.zeros_like(q_rand)
+    got, _ = run_gpu(g, gpu, store=False)
+    want = _uniform_attention_expected(g)
+    diff = (got.to(gpu).double().reshape(want.shape) - want).abs()
+    assert float((diff - (want.abs() * 2.0 ** -8 + 2e-5)).max()) <= 0.0, (
+        f"uniform attention: max-abs diff {float(diff.max()):.3e}")
+    q, want = _needle_queries(g)
+    g.q = q.reshape(q_rand.shape)
+    got, _ = run_gpu(g, gpu, store=False)
+    got = got.to(gpu).reshape(want.shape)
+    diff = (got.double() - want.double()).abs()
+    assert bool((diff <= want.double().abs() * 2.0 ** -8 + 1e-6).all()), (
+        f"needle queries: max-abs diff {float(diff.max()):.3e}")
