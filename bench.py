@@ -604,6 +604,28 @@ def run_small_launch_extends(dev, steps: int, warmup: int):
     return rows
 
 
+def run_few_long_requests_decode(dev, steps: int, warmup: int):
+    """Decode with one long request alone on the chip, or beside short ones: every workgroup's
+    partial belongs to the same request, so the merge sees up to a hundred items per row.  Not
+    one of the benchmark shapes; time per step and the rate over the K/V bytes of the step."""
+    from mini_sglang_amd.workloads import build_workload
+
+    rows = []
+    for name, lens in (("one_request_8k", [8192]), ("one_request_32k", [32768]),
+                       ("one_request_128k", [131072]),
+                       ("one_request_100k_beside_31_of_1k", [100000] + [1024] * 31)):
+        wl = build_workload(name, "decode", seed=7, n_q=32, n_kv=8, kv_lens=lens, pool_device=dev)
+        g = wl.to(dev)
+        ms, _, _ = time_steps(make_step(g), steps, warmup)
+        row = {"sizes": name, "n_q": 32, "n_kv": 8, "head_dim": 128, "us": ms * 1e3,
+               "algorithmic_bytes": wl.attention_bytes(),
+               "achieved_TBps": wl.attention_bytes() / (ms * 1e-3) / 1e12}
+        log(f"[few long requests] {name}: {row['us']:.1f} us, {row['achieved_TBps']:.2f} TB/s")
+        rows.append(row)
+        del g, wl
+    return rows
+
+
 PROBE_SRC = os.path.join(ROOT, "bench_probes.hip")
 PROBE_LIB = os.path.join(ROOT, "bench_probes.so")
 
@@ -808,6 +830,7 @@ def main():
         result["decode_step_graph"] = run_decode_step_graph(dev, args.steps, args.warmup)
         result["state_pool_copy"] = run_state_pool(dev, args.steps, args.warmup, not args.no_cpu_baseline)
         result["small_launch_extends"] = run_small_launch_extends(dev, args.steps, args.warmup)
+        result["few_long_requests_decode"] = run_few_long_requests_decode(dev, args.steps, args.warmup)
     result["all_configs"] = rows
     print(json.dumps(result))
 
