@@ -83,22 +83,7 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
   const int qblk = p.n_qblk - 1 - (seq % p.n_qblk);
   const int want_rank = pair / p.n_kv;
   const int kvh = pair - want_rank * p.n_kv;
-  __shared__ int ranked_request;
-  if (p.batch <= kRankedBatch) {
-    for (int i = tid; i < p.batch; i += NW * 64) {
-      const int len_i = p.kv_indptr[i + 1] - p.kv_indptr[i];
-      int rank = 0;
-      for (int j = 0; j < p.batch; ++j) {
-        const int len_j = p.kv_indptr[j + 1] - p.kv_indptr[j];
-        rank += (len_j > len_i) || (len_j == len_i && j < i);
-      }
-      if (rank == want_rank) ranked_request = i;
-    }
-  } else if (tid == 0) {
-    ranked_request = want_rank;  // many requests balance by their number: batch order
-  }
-  __syncthreads();
-  const int b = ranked_request;
+  const int b = request_of_rank<NW * 64>(p.kv_indptr, p.batch, want_rank, tid);
 
   const int q_start = p.qo_indptr[b];
   const int q_len = min(p.qo_indptr[b + 1] - q_start, p.max_len_extend);
@@ -712,22 +697,7 @@ __global__ __launch_bounds__(512) void prefill_pingpong_kernel(PrefillParams p) 
   const int qblk = p.n_qblk - 1 - (seq % p.n_qblk);
   const int want_rank = pair / p.n_kv;
   const int kvh = pair - want_rank * p.n_kv;
-  __shared__ int ranked_request;
-  if (p.batch <= kRankedBatch) {
-    for (int i = tid; i < p.batch; i += NW * 64) {
-      const int len_i = p.kv_indptr[i + 1] - p.kv_indptr[i];
-      int rank = 0;
-      for (int j = 0; j < p.batch; ++j) {
-        const int len_j = p.kv_indptr[j + 1] - p.kv_indptr[j];
-        rank += (len_j > len_i) || (len_j == len_i && j < i);
-      }
-      if (rank == want_rank) ranked_request = i;
-    }
-  } else if (tid == 0) {
-    ranked_request = want_rank;
-  }
-  __syncthreads();
-  const int b = ranked_request;
+  const int b = request_of_rank<NW * 64>(p.kv_indptr, p.batch, want_rank, tid);
 
   const int q_start = p.qo_indptr[b];
   const int q_len = min(p.qo_indptr[b + 1] - q_start, p.max_len_extend);

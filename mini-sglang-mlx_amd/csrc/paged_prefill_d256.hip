@@ -80,22 +80,7 @@ __global__ __launch_bounds__(kNW * 64) void prefill_tile256_kernel(PrefillParams
   const int qblk = p.n_qblk - 1 - (seq % p.n_qblk);
   const int want_rank = pair / p.n_kv;
   const int kvh = pair - want_rank * p.n_kv;
-  __shared__ int ranked_request;
-  if (p.batch <= kRankedBatch) {
-    for (int i = tid; i < p.batch; i += kNW * 64) {
-      const int len_i = p.kv_indptr[i + 1] - p.kv_indptr[i];
-      int rank = 0;
-      for (int j = 0; j < p.batch; ++j) {
-        const int len_j = p.kv_indptr[j + 1] - p.kv_indptr[j];
-        rank += (len_j > len_i) || (len_j == len_i && j < i);
-      }
-      if (rank == want_rank) ranked_request = i;
-    }
-  } else if (tid == 0) {
-    ranked_request = want_rank;  // many requests balance by their number: batch order
-  }
-  __syncthreads();
-  const int b = __builtin_amdgcn_readfirstlane(ranked_request);
+  const int b = __builtin_amdgcn_readfirstlane(request_of_rank<kNW * 64>(p.kv_indptr, p.batch, want_rank, tid));
 
   const int q_start = __builtin_amdgcn_readfirstlane(p.qo_indptr[b]);
   const int q_len = min(__builtin_amdgcn_readfirstlane(p.qo_indptr[b + 1]) - q_start, p.max_len_extend);

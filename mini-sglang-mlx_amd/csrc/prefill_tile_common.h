@@ -1,6 +1,7 @@
 // LDS-direct loads, counted waits and transposing LDS reads shared by the prefill tile kernels.
 #pragma once
 #include "msgl_device.h"
+#include "prefill_params.h"
 
 namespace msgl {
 
@@ -53,6 +54,35 @@ __device__ __forceinline__ void wait_vm_at_most() {
 __device__ __forceinline__ u32x2_t lds_read_tr16(const unsigned char* p) {
   const s16x4_t v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(MSGL_LDS_PTR(s16x4_t, p));
   return __builtin_bit_cast(u32x2_t, v);
+}
+
+// The request whose kv length has rank `want_rank` in decreasing order (ties: lower index first),
+// found by the workgroup itself: lengths into LDS once, then each thread ranks one request
+// against all of them with broadcast LDS reads.  (Ranking straight from global memory cost every
+// workgroup of a 64-request launch 3.4 us.)  Every thread of the workgroup calls it; beyond
+// kRankedBatch requests the order is the batch order.
+typedef int i32x4_t __attribute__((ext_vector_type(4)));
+template <int THREADS>
+__device__ __forceinline__ int request_of_rank(const int32_t* kv_indptr, int batch, int want_rank, int tid) {
+  if (batch > kRankedBatch) return want_rank;  // many requests balance by their number
+  __shared__ __attribute__((aligned(16))) int lens[kRankedBatch];
+  __shared__ int found;
+  const int padded = (batch + 3) & ~3;
+  for (int i = tid; i < padded; i += THREADS)
+    lens[i] = i < batch ? kv_indptr[i + 1] - kv_indptr[i] : (int)0x80000000;
+  __syncthreads();
+  for (int i = tid; i < batch; i += THREADS) {
+    const int len_i = lens[i];
+    int rank = 0;
+    for (int j = 0; j < padded; j += 4) {
+      const i32x4_t l4 = *reinterpret_cast<const i32x4_t*>(&lens[j]);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) rank += (l4[e] > len_i) || (l4[e] == len_i && j + e < i);
+    }
+    if (rank == want_rank) found = i;
+  }
+  __syncthreads();
+  return found;
 }
 
 }  // namespace msgl

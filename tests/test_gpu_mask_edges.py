@@ -33,7 +33,7 @@ def test_decode_sees_every_key_once(gpu, kv_lens):
 
 
 @pytest.mark.parametrize("is_cross,window", MASKS)
-@pytest.mark.parametrize("q_len", [1, 8])
+@pytest.mark.parametrize("q_len", [1, 8, 12, 16])
 def test_split_k_route_mask_edges(gpu, q_len, is_cross, window):
     wl = one_hot_values(build_workload(
         "e", "prefill", seed=6, n_q=16, n_kv=4, kv_lens=[q_len + 3000, q_len + 1023, q_len + 1024, q_len + 7777],

@@ -91,9 +91,10 @@ def test_tile_route_group_sizes(gpu, tile_variant, n_q, n_kv):
 
 
 @pytest.mark.parametrize("is_cross,window", MASKS)
-@pytest.mark.parametrize("q_len", [1, 3, 8])
+@pytest.mark.parametrize("q_len", [1, 3, 8, 11, 16])
 def test_splitk_route_masks(gpu, q_len, is_cross, window):
-    # short query blocks (verify / draft proposal): q_len * group <= 64
+    # short query blocks (verify / draft proposal): q_len * group <= 64; one, two and three
+    # tiles of 16 columns in a wave (q_len 3, 8, 11), four on two waves (16)
     wl = build_workload("t", "prefill", seed=300 + q_len, n_q=16, n_kv=4,
                         kv_lens=[q_len, 40 + q_len, 333 + q_len, 1500 + q_len],
                         extend_lens=[q_len] * 4, pool_factor=1.3, store_new=True,
