@@ -74,13 +74,12 @@ __global__ __launch_bounds__(NW * 64) void prefill_tile_kernel(PrefillParams p) 
   // in id order, so long requests start first and short ones fill the tail); each block
   // finds "the request of rank r" itself from kv_indptr, the host never sees the lengths.
   // Beyond kRankedBatch requests the order is the batch order.
-  const int xcd = blockIdx.x & 7;
-  const int seq = blockIdx.x >> 3;
-  const int unit = (seq / p.n_qblk) * 8 + xcd;  // (request, kv head, key split)
-  if (unit >= p.n_pairs * p.n_ksplit) return;
+  const BlockWork work = prefill_block_work(p);
+  if (!work.ok) return;
+  const int unit = work.unit;  // (request, kv head, key split)
   const int pair = unit / p.n_ksplit;
   const int split = unit - pair * p.n_ksplit;
-  const int qblk = p.n_qblk - 1 - (seq % p.n_qblk);
+  const int qblk = work.qblk;
   const int want_rank = pair / p.n_kv;
   const int kvh = pair - want_rank * p.n_kv;
   const int b = request_of_rank<NW * 64>(p.kv_indptr, p.batch, want_rank, tid);
@@ -688,13 +687,12 @@ __global__ __launch_bounds__(512) void prefill_pingpong_kernel(PrefillParams p) 
   const int c32 = lane & 31;
 
   // ---- block -> (request, kv head, key split, q block): as in prefill_tile_kernel ----------
-  const int xcd = blockIdx.x & 7;
-  const int seq = blockIdx.x >> 3;
-  const int unit = (seq / p.n_qblk) * 8 + xcd;
-  if (unit >= p.n_pairs * p.n_ksplit) return;
+  const BlockWork work = prefill_block_work(p);
+  if (!work.ok) return;
+  const int unit = work.unit;  // (request, kv head, key split)
   const int pair = unit / p.n_ksplit;
   const int split = unit - pair * p.n_ksplit;
-  const int qblk = p.n_qblk - 1 - (seq % p.n_qblk);
+  const int qblk = work.qblk;
   const int want_rank = pair / p.n_kv;
   const int kvh = pair - want_rank * p.n_kv;
   const int b = request_of_rank<NW * 64>(p.kv_indptr, p.batch, want_rank, tid);

@@ -71,13 +71,12 @@ __global__ __launch_bounds__(kNW * 64) void prefill_tile256_kernel(PrefillParams
   // XCDs, the q blocks of one (request, kv head, key split) read the same keys, share an XCD and
   // run heaviest first, requests in order of decreasing kv length (each block ranks the requests
   // itself from kv_indptr)
-  const int xcd = blockIdx.x & 7;
-  const int seq = blockIdx.x >> 3;
-  const int unit = (seq / p.n_qblk) * 8 + xcd;  // (request, kv head, key split)
-  if (unit >= p.n_pairs * p.n_ksplit) return;
+  const BlockWork work = prefill_block_work(p);
+  if (!work.ok) return;
+  const int unit = work.unit;  // (request, kv head, key split)
   const int pair = unit / p.n_ksplit;
   const int split = unit - pair * p.n_ksplit;
-  const int qblk = p.n_qblk - 1 - (seq % p.n_qblk);
+  const int qblk = work.qblk;
   const int want_rank = pair / p.n_kv;
   const int kvh = pair - want_rank * p.n_kv;
   const int b = __builtin_amdgcn_readfirstlane(request_of_rank<kNW * 64>(p.kv_indptr, p.batch, want_rank, tid));

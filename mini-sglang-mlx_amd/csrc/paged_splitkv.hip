@@ -157,6 +157,7 @@ __device__ __forceinline__ bool locate_segment(const SplitKvParams& p, int seg, 
     incl = wave_inclusive_scan(n);
     total += __shfl(incl, kWave - 1, kWave);
   }
+  total = max(total - p.boundary, 0);  // nothing follows the last request: its empty positions go
   const int len = segment_length(total, p.n_seg, p.min_seg);
   *seg_len = len;
   *total_out = total;
@@ -774,10 +775,13 @@ void splitkv_set_boundary(int v) { t_boundary = v; }
 // A boundary costs a workgroup about 8 us (measured on the benchmark shapes, one and eight
 // queries per request); in that time it would stream 8 us x (what the chip reads per us) /
 // (workgroups x bytes of one token's K and V rows for the workgroup's kv heads) tokens.
+// A workgroup with the chip to itself streams about 40 GB/s (its own chain of loads, not the
+// memory system, is the limit), so a small launch charges what one workgroup reads in that time.
 static int boundary_tokens(int64_t n_wgs, int nwh, int64_t head_dim) {
   if (t_boundary != 0) return t_boundary > 0 ? (t_boundary < 4096 ? t_boundary : 4096) : 0;
   const double bytes_per_token = (double)nwh * 2.0 * (double)head_dim * 2.0;
-  const double tokens = 8.0 * 6.2e6 / ((double)(n_wgs > 0 ? n_wgs : 1) * bytes_per_token);
+  const double wg_bytes_per_us = std::min(6.2e6 / (double)(n_wgs > 0 ? n_wgs : 1), 40e3);
+  const double tokens = 8.0 * wg_bytes_per_us / bytes_per_token;
   const int64_t t = ((int64_t)tokens + 8) / 16 * 16;
   return (int)(t < 0 ? 0 : (t > 1024 ? 1024 : t));
 }

@@ -16,6 +16,7 @@ struct PrefillParams {
   int64_t k_stride0, v_stride0;
   int32_t batch, n_q, n_kv, group;
   int32_t n_qblk, n_pairs;  // q blocks per (request, kv head); batch * n_kv
+  int32_t xcds_per_unit;    // see prefill_xcds_per_unit()
   int32_t max_len_extend, is_cross, window;
   float scale_log2e;
   uint32_t max_slot;  // num_slots - 1: slot ids are clamped to it before they become addresses
@@ -47,6 +48,20 @@ inline int prefill_block_rows(int64_t head_dim) {
   return head_dim == 256 ? kPrefillBlockRows256 : kPrefillBlockRows;
 }
 
+// Workgroup ids go round the 8 XCDs.  A (request, kv head, key split) unit normally keeps all its
+// query blocks on one XCD (they read the same keys: one L2 holds them); with fewer than 8 units
+// that would leave XCDs without work (a single request with 2 kv heads: 6 of 8), so each unit
+// then spreads its query blocks over 8 / (units rounded up to a power of two) XCDs.
+inline int prefill_xcds_per_unit(int64_t n_units) {
+  if (n_units >= 5 || n_units <= 0) return 1;
+  return n_units <= 1 ? 8 : (n_units <= 2 ? 4 : 2);
+}
+// workgroups on the busiest XCD
+inline int64_t prefill_blocks_per_xcd(int64_t n_units, int64_t n_qblk) {
+  const int x = prefill_xcds_per_unit(n_units);
+  return x > 1 ? (n_qblk + x - 1) / x : (n_units + 7) / 8 * n_qblk;
+}
+
 // Number of key splits for a launch, from sizes the host knows (the per-request lengths stay on
 // the device: the average visible length stands for all of them).  Cost model: the (request, kv
 // head, split) units are dealt round-robin to the 8 XCDs, a unit brings its query blocks, and an
@@ -62,7 +77,7 @@ inline int prefill_key_splits(int64_t batch, int64_t total_kv, int64_t n_kv, int
   const int64_t n_qblk = (max_len_extend * group + block_rows - 1) / block_rows;
   const int64_t pairs = batch * n_kv;
   auto rounds = [&](int64_t k) {
-    const int64_t blocks = (pairs * k + kXcds - 1) / kXcds * n_qblk;  // on the busiest XCD
+    const int64_t blocks = prefill_blocks_per_xcd(pairs * k, n_qblk);  // on the busiest XCD
     return (blocks + kUnitsPerXcd - 1) / kUnitsPerXcd;
   };
   if (n_qblk <= 0 || rounds(1) > 4) return 1;
@@ -121,7 +136,8 @@ inline int make_prefill_params(const PrefillArgs& a, PrefillParams& p, int64_t& 
   const int64_t rows = (int64_t)a.max_len_extend * p.group;
   const int64_t n_qblk = (rows + block_rows - 1) / block_rows;
   const int64_t n_pairs = a.batch * a.n_kv;
-  n_blocks = (n_pairs * p.n_ksplit + 7) / 8 * 8 * n_qblk;
+  p.xcds_per_unit = prefill_xcds_per_unit(n_pairs * p.n_ksplit);
+  n_blocks = 8 * prefill_blocks_per_xcd(n_pairs * p.n_ksplit, n_qblk);
   if (n_qblk <= 0 || n_blocks <= 0) {
     n_blocks = 0;
     return MSGL_OK;

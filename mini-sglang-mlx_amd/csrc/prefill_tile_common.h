@@ -61,6 +61,31 @@ __device__ __forceinline__ u32x2_t lds_read_tr16(const unsigned char* p) {
 // against all of them with broadcast LDS reads.  (Ranking straight from global memory cost every
 // workgroup of a 64-request launch 3.4 us.)  Every thread of the workgroup calls it; beyond
 // kRankedBatch requests the order is the batch order.
+// Workgroup id -> (unit = (request rank, kv head, key split), query block), heaviest query block
+// (latest rows) first; `ok` is false for the ids that pad the grid.  Consecutive ids go to
+// different XCDs.
+struct BlockWork {
+  int unit, qblk;
+  bool ok;
+};
+__device__ __forceinline__ BlockWork prefill_block_work(const PrefillParams& p) {
+  const int xcd = blockIdx.x & 7;
+  const int seq = blockIdx.x >> 3;
+  BlockWork w;
+  if (p.xcds_per_unit > 1) {  // few units: each spreads its query blocks over several XCDs
+    const int side_by_side = 8 / p.xcds_per_unit;
+    w.unit = xcd % side_by_side;
+    const int j = seq * p.xcds_per_unit + xcd / side_by_side;
+    w.qblk = p.n_qblk - 1 - j;
+    w.ok = w.unit < p.n_pairs * p.n_ksplit && j < p.n_qblk;
+  } else {  // all query blocks of a unit on one XCD, issued back to back
+    w.unit = (seq / p.n_qblk) * 8 + xcd;
+    w.qblk = p.n_qblk - 1 - (seq % p.n_qblk);
+    w.ok = w.unit < p.n_pairs * p.n_ksplit;
+  }
+  return w;
+}
+
 typedef int i32x4_t __attribute__((ext_vector_type(4)));
 template <int THREADS>
 __device__ __forceinline__ int request_of_rank(const int32_t* kv_indptr, int batch, int want_rank, int tid) {
