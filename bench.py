@@ -41,7 +41,7 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def time_steps(fn, steps: int, warmup: int):
+def time_steps(fn, steps: int, warmup: int, spinup_ms: float = SPINUP_MS):
     """`warmup` untimed steps, then exactly `steps` back-to-back steps between two HIP events
     recorded on torch's current stream (the stream every operator launches on), bracketed by
     device syncs: that mean is the reported figure.  Two diagnostic passes follow: one that
@@ -73,7 +73,7 @@ def time_steps(fn, steps: int, warmup: int):
         spin1 = torch.cuda.Event(enable_timing=True)
         spin1.record()
         spin1.synchronize()
-        if spin0.elapsed_time(spin1) >= SPINUP_MS:
+        if spin0.elapsed_time(spin1) >= spinup_ms:
             break
     for _ in range(warmup):
         fn()
@@ -626,6 +626,36 @@ def run_few_long_requests_decode(dev, steps: int, warmup: int):
     return rows
 
 
+def run_reference_microbench_shapes(dev, steps: int, warmup: int):
+    """The shapes of the reference's own micro-benchmarks (one sequence, head_dim 256, its four
+    head configurations, nine lengths: `test_and_bench/paged_prefill_attention.py:18-25, 267` with
+    prefix 0, `paged_decode_attention.py:17-24, 288`), in microseconds per call.  The reference
+    prints these beside MLX's dense SDPA and ships no recorded output, so there is no ratio to
+    quote: the numbers are here for whoever runs the reference's scripts on their own machine."""
+    from mini_sglang_amd.workloads import build_workload
+
+    lens = (1, 237, 512, 809, 1024, 2048, 3333, 4096, 8192)
+    rows = []
+    for kind in ("prefill", "decode"):
+        for n_kv, n_q in ((2, 16), (4, 16), (4, 24), (2, 32)):
+            us = []
+            for length in lens:
+                wl = build_workload("m", kind, seed=7, n_q=n_q, n_kv=n_kv, head_dim=256,
+                                    kv_lens=[length],
+                                    extend_lens=[length] if kind == "prefill" else None,
+                                    pool_device=dev)
+                g = wl.to(dev)
+                ms, _, _ = time_steps(make_step(g), max(3, steps // 2), max(1, warmup // 2),
+                                      spinup_ms=10.0)
+                us.append(round(ms * 1e3, 1))
+                del g, wl
+            rows.append({"kind": kind, "head_dim": 256, "n_kv": n_kv, "n_q": n_q,
+                         "lengths": list(lens), "us": us})
+            log(f"[reference shapes] {kind} kv {n_kv} q {n_q}: " +
+                "  ".join(f"{n}:{u}" for n, u in zip(lens, us)))
+    return rows
+
+
 PROBE_SRC = os.path.join(ROOT, "bench_probes.hip")
 PROBE_LIB = os.path.join(ROOT, "bench_probes.so")
 
@@ -831,6 +861,7 @@ def main():
         result["state_pool_copy"] = run_state_pool(dev, args.steps, args.warmup, not args.no_cpu_baseline)
         result["small_launch_extends"] = run_small_launch_extends(dev, args.steps, args.warmup)
         result["few_long_requests_decode"] = run_few_long_requests_decode(dev, args.steps, args.warmup)
+        result["reference_microbench_shapes"] = run_reference_microbench_shapes(dev, args.steps, args.warmup)
     result["all_configs"] = rows
     print(json.dumps(result))
 
