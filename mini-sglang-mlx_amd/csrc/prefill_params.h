@@ -48,18 +48,21 @@ inline int prefill_block_rows(int64_t head_dim) {
   return head_dim == 256 ? kPrefillBlockRows256 : kPrefillBlockRows;
 }
 
-// Workgroup ids go round the 8 XCDs.  A (request, kv head, key split) unit normally keeps all its
-// query blocks on one XCD (they read the same keys: one L2 holds them); with fewer than 8 units
-// that would leave XCDs without work (a single request with 2 kv heads: 6 of 8), so each unit
-// then spreads its query blocks over 8 / (units rounded up to a power of two) XCDs.
+// Workgroup ids go round the 8 XCDs.  A (request, kv head, key split) unit keeps all its query
+// blocks on one XCD (they read the same keys: one L2 holds them), so units are dealt to the XCDs
+// eight at a time.  The units left over when their number is no multiple of 8 would leave XCDs
+// without work (a single request with 2 kv heads: 6 of 8), so up to 4 left-over units spread
+// their query blocks over 8 / (their number rounded up to a power of two) XCDs each.
 inline int prefill_xcds_per_unit(int64_t n_units) {
-  if (n_units >= 5 || n_units <= 0) return 1;
-  return n_units <= 1 ? 8 : (n_units <= 2 ? 4 : 2);
+  const int64_t left = n_units % 8;
+  if (left == 0 || left >= 5) return 1;
+  return left == 1 ? 8 : (left == 2 ? 4 : 2);
 }
 // workgroups on the busiest XCD
 inline int64_t prefill_blocks_per_xcd(int64_t n_units, int64_t n_qblk) {
   const int x = prefill_xcds_per_unit(n_units);
-  return x > 1 ? (n_qblk + x - 1) / x : (n_units + 7) / 8 * n_qblk;
+  const int64_t last_row = n_units % 8 == 0 ? 0 : (n_qblk + x - 1) / x;
+  return n_units / 8 * n_qblk + last_row;
 }
 
 // Number of key splits for a launch, from sizes the host knows (the per-request lengths stay on

@@ -71,17 +71,20 @@ struct BlockWork {
 __device__ __forceinline__ BlockWork prefill_block_work(const PrefillParams& p) {
   const int xcd = blockIdx.x & 7;
   const int seq = blockIdx.x >> 3;
+  const int n_units = p.n_pairs * p.n_ksplit;
+  const int whole_rows = n_units >> 3;  // rows of 8 units, one unit per XCD
   BlockWork w;
-  if (p.xcds_per_unit > 1) {  // few units: each spreads its query blocks over several XCDs
-    const int side_by_side = 8 / p.xcds_per_unit;
-    w.unit = xcd % side_by_side;
-    const int j = seq * p.xcds_per_unit + xcd / side_by_side;
-    w.qblk = p.n_qblk - 1 - j;
-    w.ok = w.unit < p.n_pairs * p.n_ksplit && j < p.n_qblk;
-  } else {  // all query blocks of a unit on one XCD, issued back to back
+  if (seq < whole_rows * p.n_qblk) {  // all query blocks of a unit on one XCD, back to back
     w.unit = (seq / p.n_qblk) * 8 + xcd;
     w.qblk = p.n_qblk - 1 - (seq % p.n_qblk);
-    w.ok = w.unit < p.n_pairs * p.n_ksplit;
+    w.ok = true;
+  } else {  // the left-over units: each on xcds_per_unit XCDs
+    const int side_by_side = 8 / p.xcds_per_unit;
+    const int u = xcd % side_by_side;
+    const int j = (seq - whole_rows * p.n_qblk) * p.xcds_per_unit + xcd / side_by_side;
+    w.unit = whole_rows * 8 + u;
+    w.qblk = p.n_qblk - 1 - j;
+    w.ok = w.unit < n_units && j < p.n_qblk;
   }
   return w;
 }
