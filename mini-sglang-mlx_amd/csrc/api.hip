@@ -45,11 +45,16 @@ int32_t segments(int64_t total_kv, int64_t n_kv, int64_t head_dim, int64_t cols)
   if (t >= 1) return (int32_t)(t < (1 << 20) ? t : (1 << 20));
   return msgl::splitkv_default_segments(total_kv, n_kv, head_dim, cols, min_segment());
 }
-int64_t smallq_max_cols() {
+// Largest q_len * group that takes the split-K route.  Default at head_dim 128: 48 (up to three
+// column tiles in one wave); 49-64 columns would run on two waves per kv head that each read
+// every K / V row, and the tile kernel with ragged key shares is as fast or faster on them.
+// head_dim 256 keeps every short query block on the split-K kernel (its tile kernel has no
+// ragged shares, and uniform ones make one long request among short ones 4-6 x slower).
+int64_t smallq_max_cols(int64_t head_dim) {
   const int64_t t = t_tune[MSGL_TUNE_SMALLQ_MAXCOLS];
   if (t < 0) return 0;  // negative: never take the split-K route
   if (t > 0) return t < msgl::kSplitKvMaxCols ? t : msgl::kSplitKvMaxCols;
-  return msgl::kSplitKvMaxCols;
+  return head_dim == 128 ? 48 : msgl::kSplitKvMaxCols;
 }
 
 }  // namespace
@@ -218,8 +223,17 @@ int msgl_paged_decode_attention_noalloc(const void* q, const void* k_cache, cons
                           k_cache_stride0, v_cache_stride0, sm_scale, max_kv_splits, dtype, stream);
 }
 
-static bool use_splitkv_route(int64_t group, int64_t max_len_extend) {
-  return max_len_extend >= 1 && group * max_len_extend <= smallq_max_cols();
+// Ragged key shares for the tile kernels (one query block per (request, kv head)): head_dim 128
+// with the ping-pong kernel only for now.
+static int ragged_tiles(int64_t batch, int64_t total_kv, int64_t n_kv, int64_t group,
+                        int64_t max_len_extend, int64_t head_dim) {
+  if (head_dim != 128 || msgl::tile_variant() != 0) return 0;
+  return msgl::prefill_ragged_tiles(batch, total_kv, n_kv, group, max_len_extend,
+                                    msgl::prefill_block_rows(head_dim), t_key_splits);
+}
+
+static bool use_splitkv_route(int64_t group, int64_t max_len_extend, int64_t head_dim) {
+  return max_len_extend >= 1 && group * max_len_extend <= smallq_max_cols(head_dim);
 }
 // Longer queries run the MFMA tile kernels.  The older route for head_dim 256, the split-K
 // kernel once per chunk of queries (each launch re-reads the visible keys), is kept behind
@@ -228,7 +242,7 @@ static bool use_chunked_route(int64_t head_dim, int64_t group) {
   return head_dim == 256 && msgl::tile_variant() == 2 && group <= msgl::kSplitKvMaxCols;
 }
 static int32_t chunk_queries(int64_t group) {
-  return (int32_t)std::max<int64_t>(1, std::min<int64_t>(smallq_max_cols(), msgl::kSplitKvMaxCols) / group);
+  return (int32_t)std::max<int64_t>(1, std::min<int64_t>(smallq_max_cols(256), msgl::kSplitKvMaxCols) / group);
 }
 
 size_t msgl_paged_prefill_workspace_bytes(int64_t batch, int64_t total_q, int64_t total_kv,
@@ -238,10 +252,14 @@ size_t msgl_paged_prefill_workspace_bytes(int64_t batch, int64_t total_q, int64_
       num_q_heads % num_kv_heads != 0)
     return 0;
   const int64_t group = num_q_heads / num_kv_heads;
-  if (!use_splitkv_route(group, max_len_extend)) {
+  if (!use_splitkv_route(group, max_len_extend, head_dim)) {
     if (!use_chunked_route(head_dim, group)) {
       // tile kernels: partials of a key split, if this launch would use one (a sliding window,
       // unknown here, can only lower the count)
+      const int ragged = ragged_tiles(batch, total_kv, num_kv_heads, group, max_len_extend, head_dim);
+      if (ragged > 0)
+        return msgl::prefill_ragged_workspace_bytes(batch, total_kv, num_kv_heads, group,
+                                                    max_len_extend, head_dim, ragged);
       const int k = msgl::prefill_key_splits(batch, total_kv, num_kv_heads, group, max_len_extend, 0,
                                              msgl::prefill_block_rows(head_dim), t_key_splits);
       return msgl::prefill_split_workspace_bytes(total_q, num_q_heads, head_dim, k);
@@ -278,7 +296,7 @@ int msgl_paged_prefill_attention(const void* q, const void* k_cache, const void*
     return MSGL_ERR_NULL_POINTER;
   const int64_t group = num_q_heads / num_kv_heads;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const bool direct = use_splitkv_route(group, max_len_extend);
+  const bool direct = use_splitkv_route(group, max_len_extend, head_dim);
   if (direct || use_chunked_route(head_dim, group)) {
     const int32_t per_launch = direct ? max_len_extend : chunk_queries(group);
     const int32_t n_seg = segments(total_kv, num_kv_heads, head_dim, group * per_launch);
@@ -340,9 +358,19 @@ int msgl_paged_prefill_attention(const void* q, const void* k_cache, const void*
   a.max_len_extend = max_len_extend;
   a.is_cross = is_cross_attention ? 1 : 0;
   a.window = sliding_window_size;
-  a.key_splits = msgl::prefill_key_splits(batch, total_kv, num_kv_heads, group, max_len_extend,
-                                          sliding_window_size, msgl::prefill_block_rows(head_dim),
-                                          t_key_splits);
+  a.key_splits = 1;
+  a.ragged_tiles = ragged_tiles(batch, total_kv, num_kv_heads, group, max_len_extend, head_dim);
+  if (a.ragged_tiles > 0) {
+    // ragged shares need room for their partials; without it the keys go in one pass
+    const size_t need = msgl::prefill_ragged_workspace_bytes(batch, total_kv, num_kv_heads, group,
+                                                             max_len_extend, head_dim, a.ragged_tiles);
+    if (need > 0 && (!workspace || workspace_bytes < need || !aligned16(workspace))) a.ragged_tiles = 0;
+    else a.workspace = workspace;
+  } else {
+    a.key_splits = msgl::prefill_key_splits(batch, total_kv, num_kv_heads, group, max_len_extend,
+                                            sliding_window_size, msgl::prefill_block_rows(head_dim),
+                                            t_key_splits);
+  }
   if (a.key_splits > 1) {
     // the split is an optimisation: without room for its partials the keys go in one pass
     const size_t need = msgl::prefill_split_workspace_bytes(total_q, num_q_heads, head_dim, a.key_splits);

@@ -76,6 +76,9 @@ struct PrefillArgs {
   // key_splits * total_q * n_q * (head_dim + 1) floats
   int32_t key_splits;
   void* workspace;
+  // ragged shares instead (one query block per (request, kv head) only): key tiles per share,
+  // 0 = off; `workspace` then holds prefill_ragged_workspace_bytes()
+  int32_t ragged_tiles;
 };
 int launch_prefill_tile(const PrefillArgs& a, hipStream_t stream);     // head_dim 128
 // ---- paged_prefill_d256.hip ----------------------------------------------------------

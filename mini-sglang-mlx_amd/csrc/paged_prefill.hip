@@ -686,16 +686,36 @@ __global__ __launch_bounds__(512) void prefill_pingpong_kernel(PrefillParams p) 
   const int h = lane >> 5;
   const int c32 = lane & 31;
 
-  // ---- block -> (request, kv head, key split, q block): as in prefill_tile_kernel ----------
-  const BlockWork work = prefill_block_work(p);
-  if (!work.ok) return;
-  const int unit = work.unit;  // (request, kv head, key split)
-  const int pair = unit / p.n_ksplit;
-  const int split = unit - pair * p.n_ksplit;
-  const int qblk = work.qblk;
-  const int want_rank = pair / p.n_kv;
-  const int kvh = pair - want_rank * p.n_kv;
-  const int b = request_of_rank<NW * 64>(p.kv_indptr, p.batch, want_rank, tid);
+  // ---- block -> (request, kv head, key split, q block): as in prefill_tile_kernel; with ragged
+  // shares, block -> (unit = (request, share), kv head) ----------------------------------------
+  int b, kvh, split, qblk, n_shares = 1;
+  bool to_partial = p.n_ksplit > 1;  // leave a partial for the merge kernel, not the result
+  int64_t part_at = 0;               // partial row of the block's row 0 (ragged shares)
+  if (p.ragged_tiles > 0) {
+    kvh = (int)(blockIdx.x % (unsigned)p.n_kv);
+    const int u = (int)(blockIdx.x / (unsigned)p.n_kv);
+    const RaggedUnit ru = ragged_unit<NW * 64>(p, u, tid);
+    if (!ru.ok) return;
+    b = ru.request;
+    split = ru.share;
+    qblk = 0;
+    n_shares = ru.count;
+    to_partial = ru.count > 1;
+    part_at = ((int64_t)u * p.n_kv + kvh) * p.ragged_rows;
+    if (ru.share == 0 && kvh == 0 && tid == 0 && p.req_units != nullptr) {
+      p.req_units[2 * b] = ru.first;  // tells the merge kernel where the request's partials are
+      p.req_units[2 * b + 1] = ru.count;
+    }
+  } else {
+    const BlockWork work = prefill_block_work(p);
+    if (!work.ok) return;
+    const int pair = work.unit / p.n_ksplit;  // unit = (request, kv head, key split)
+    split = work.unit - pair * p.n_ksplit;
+    qblk = work.qblk;
+    const int want_rank = pair / p.n_kv;
+    kvh = pair - want_rank * p.n_kv;
+    b = request_of_rank<NW * 64>(p.kv_indptr, p.batch, want_rank, tid);
+  }
 
   const int q_start = p.qo_indptr[b];
   const int q_len = min(p.qo_indptr[b + 1] - q_start, p.max_len_extend);
@@ -713,7 +733,12 @@ __global__ __launch_bounds__(512) void prefill_pingpong_kernel(PrefillParams p) 
   int k_lo = (p.window > 0) ? max(0, prefix + qi_lo - p.window + 1) : 0;
   k_lo &= ~(kBN - 1);
   if (k_hi < k_lo) k_hi = k_lo;
-  if (p.n_ksplit > 1) {
+  if (p.ragged_tiles > 0) {  // the request's shares are equal: none longer than ragged_tiles
+    const int all_tiles = (k_hi - k_lo + kBN - 1) / kBN;
+    const int share = (all_tiles + n_shares - 1) / n_shares * kBN;
+    k_lo = min(k_lo + split * share, k_hi);
+    k_hi = min(k_hi, k_lo + share);
+  } else if (p.n_ksplit > 1) {
     const int all_tiles = (k_hi - k_lo + kBN - 1) / kBN;
     const int share = (all_tiles + p.n_ksplit - 1) / p.n_ksplit * kBN;
     k_lo = min(k_lo + split * share, k_hi);
@@ -1093,12 +1118,13 @@ __global__ __launch_bounds__(512) void prefill_pingpong_kernel(PrefillParams p) 
   float l = l_run;
   l += __shfl_xor(l, 32, kWave);
   const float inv = (l > 0.f) ? 1.0f / l : 0.f;
-  if (p.n_ksplit > 1) {
+  if (to_partial) {
     const int row = row0 + w * 32 + c32;
     if (row < rows_total) {
       const int qi = row / p.group;
       const int hh = row - qi * p.group;
-      const int64_t at = (int64_t)split * p.part_rows + (int64_t)(q_start + qi) * p.n_q + kvh * p.group + hh;
+      const int64_t at = p.ragged_tiles > 0 ? part_at + row
+                                            : (int64_t)split * p.part_rows + (int64_t)(q_start + qi) * p.n_q + kvh * p.group + hh;
       if (h == 0) p.part_lse[at] = (l > 0.f) ? m_run + __log2f(l) : kNegInf;
       float* dst = p.part_o + at * D + 4 * h;
 #pragma unroll
@@ -1187,11 +1213,67 @@ __global__ __launch_bounds__(256) void prefill_merge_kernel(const float* __restr
   }
 }
 
+// The same for ragged shares: request b's partials are units req_units[2 b] .. + req_units[2 b + 1],
+// each [kv head][row of the block]; a request with one share was written by the attention kernel.
+template <int D>
+__global__ __launch_bounds__(256) void prefill_ragged_merge_kernel(PrefillParams p) {
+  constexpr int V = D / 32;  // dims per lane
+  const int b = blockIdx.y;
+  const int q_start = p.qo_indptr[b];
+  const int q_len = min(p.qo_indptr[b + 1] - q_start, p.max_len_extend);
+  const int64_t r = (int64_t)blockIdx.x * 8 + (threadIdx.x >> 5);  // row of the request, token-major
+  if (r >= (int64_t)q_len * p.n_q) return;
+  const int first = p.req_units[2 * b];
+  const int count = p.req_units[2 * b + 1];
+  if (count <= 1) return;
+  const int qi = (int)(r / p.n_q);
+  const int hq = (int)(r - (int64_t)qi * p.n_q);
+  const int kvh = hq / p.group;
+  const int local = qi * p.group + (hq - kvh * p.group);
+  const int64_t step = (int64_t)p.n_kv * p.ragged_rows;  // partial rows from one unit to the next
+  const int64_t at0 = ((int64_t)first * p.n_kv + kvh) * p.ragged_rows + local;
+  const int c = threadIdx.x & 31;
+  float top = kNegInf;
+  for (int s = 0; s < count; ++s) top = fmaxf(top, p.part_lse[at0 + s * step]);
+  float acc[V];
+#pragma unroll
+  for (int i = 0; i < V; ++i) acc[i] = 0.f;
+  float total = 0.f;
+  for (int s = 0; s < count; ++s) {
+    const float lse = p.part_lse[at0 + s * step];
+    if (lse == kNegInf) continue;  // that share saw no key of this row
+    const float wgt = exp2f(lse - top);
+    total += wgt;
+    const float* src = p.part_o + (at0 + s * step) * D + c * V;
+#pragma unroll
+    for (int i = 0; i < V; i += 4) {
+      const f32x4_t x = *reinterpret_cast<const f32x4_t*>(src + i);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc[i + e] += wgt * x[e];
+    }
+  }
+  const float inv = (total > 0.f) ? 1.0f / total : 0.f;
+  uint16_t* dst = p.out + ((int64_t)q_start * p.n_q + r) * D + c * V;
+#pragma unroll
+  for (int i = 0; i < V; i += 4) {
+    u32x2_t wv;
+    wv[0] = pack_bf16x2(acc[i] * inv, acc[i + 1] * inv);
+    wv[1] = pack_bf16x2(acc[i + 2] * inv, acc[i + 3] * inv);
+    *reinterpret_cast<u32x2_t*>(dst + i) = wv;
+  }
+}
+
 }  // namespace
 
 int launch_prefill_merge(const PrefillParams& p, int head_dim, hipStream_t stream) {
   const int64_t rows = (int64_t)p.max_len_extend * p.n_q;
   const dim3 grid((unsigned)((rows + 7) / 8), (unsigned)p.batch);
+  if (p.ragged_tiles > 0) {
+    if (p.req_units == nullptr) return MSGL_OK;  // no request can have a second share
+    if (head_dim == 256) hipLaunchKernelGGL((prefill_ragged_merge_kernel<256>), grid, dim3(256), 0, stream, p);
+    else hipLaunchKernelGGL((prefill_ragged_merge_kernel<128>), grid, dim3(256), 0, stream, p);
+    return check_launch();
+  }
   if (head_dim == 256)
     hipLaunchKernelGGL((prefill_merge_kernel<256>), grid, dim3(256), 0, stream, p.part_o, p.part_lse,
                        p.qo_indptr, p.out, p.part_rows, p.n_q, p.n_ksplit, p.max_len_extend);
@@ -1211,7 +1293,9 @@ int launch_prefill_tile(const PrefillArgs& a, hipStream_t stream) {
   PrefillParams p;
   int64_t n_blocks = 0;
   bool wide = false;
-  const int rc = make_prefill_params(a, p, n_blocks, wide);
+  PrefillArgs args = a;
+  if (tile_variant() != 0) args.ragged_tiles = 0;  // the fused kernels know uniform key splits only
+  const int rc = make_prefill_params(args, p, n_blocks, wide);
   if (rc != MSGL_OK || n_blocks == 0) return rc;
   const dim3 grid((unsigned)n_blocks);
   if (tile_variant() == 1) {
@@ -1225,7 +1309,7 @@ int launch_prefill_tile(const PrefillArgs& a, hipStream_t stream) {
     else hipLaunchKernelGGL((prefill_pingpong_kernel<false>), grid, dim3(512), 0, stream, p);
   }
   const int launched = check_launch();
-  if (launched != MSGL_OK || p.n_ksplit == 1) return launched;
+  if (launched != MSGL_OK || (p.n_ksplit == 1 && p.ragged_tiles == 0)) return launched;
   return launch_prefill_merge(p, 128, stream);
 }
 

@@ -26,6 +26,11 @@ struct PrefillParams {
   int64_t part_rows;  // total_q * n_q: rows of one split's partial
   float* part_o;      // [n_ksplit][part_rows][head_dim]
   float* part_lse;    // [n_ksplit][part_rows]
+  // ragged shares (see prefill_ragged_tiles()): a request's keys in shares of `ragged_tiles` tiles,
+  // as many as it needs; partials are then [unit][kv head][row of the block], a unit being one
+  // (request, share), and req_units[2 b], [2 b + 1] = request b's first unit and unit count
+  int32_t ragged_tiles, ragged_units, ragged_rows;
+  int32_t* req_units;
 };
 
 constexpr int kBN = 64;  // keys per tile
@@ -100,6 +105,42 @@ inline int prefill_key_splits(int64_t batch, int64_t total_kv, int64_t n_kv, int
   return best;
 }
 
+// Ragged shares, for launches with one query block per (request, kv head) (short query blocks:
+// their cost is reading the keys).  Cutting every request's keys the same number of times makes
+// the workgroups of a long request long; instead a share is `tiles` key tiles for every request,
+// a request gets as many shares as it needs, and the workgroups find their (request, share) by a
+// prefix sum over the requests' share counts, so the grid holds no empty workgroups beyond the
+// rounding.  tiles = what gives about one workgroup per compute unit, at least kRaggedMinTiles.
+// Returns 0 when the launch does not qualify.
+constexpr int kRaggedMaxBatch = 128;  // every workgroup scans the share counts of all requests
+constexpr int kRaggedMinTiles = 16;
+inline int64_t prefill_tiles_bound(int64_t batch, int64_t total_kv) {
+  return (total_kv + kBN - 1) / kBN + 2 * batch;  // sum over requests of their key tiles, at most
+}
+inline int prefill_ragged_tiles(int64_t batch, int64_t total_kv, int64_t n_kv, int64_t group,
+                                int64_t max_len_extend, int block_rows, int64_t forced_splits) {
+  if (forced_splits > 0 || batch <= 0 || batch > kRaggedMaxBatch) return 0;
+  if (max_len_extend * group > block_rows) return 0;
+  int64_t t = (prefill_tiles_bound(batch, total_kv) * n_kv + kComputeUnits - 1) / kComputeUnits;
+  if (t < kRaggedMinTiles) t = kRaggedMinTiles;
+  return (int)(t < (1 << 20) ? t : (1 << 20));
+}
+// (request, share) units a launch can have at most
+inline int64_t prefill_ragged_units(int64_t batch, int64_t total_kv, int tiles) {
+  return prefill_tiles_bound(batch, total_kv) / tiles + batch;
+}
+// no request can need a second share: nothing to merge, no workspace
+inline bool prefill_ragged_never_splits(int64_t batch, int64_t total_kv, int tiles) {
+  return prefill_tiles_bound(batch, total_kv) <= tiles;
+}
+inline size_t prefill_ragged_workspace_bytes(int64_t batch, int64_t total_kv, int64_t n_kv, int64_t group,
+                                             int64_t max_len_extend, int64_t head_dim, int tiles) {
+  if (tiles <= 0 || prefill_ragged_never_splits(batch, total_kv, tiles)) return 0;
+  const size_t rows = (size_t)prefill_ragged_units(batch, total_kv, tiles) * (size_t)n_kv *
+                      (size_t)(max_len_extend * group);
+  return rows * (size_t)(head_dim + 1) * sizeof(float) + (size_t)batch * 2 * sizeof(int32_t);
+}
+
 inline size_t prefill_split_workspace_bytes(int64_t total_q, int64_t n_q, int64_t head_dim, int n_ksplit) {
   if (n_ksplit <= 1) return 0;
   return (size_t)n_ksplit * (size_t)total_q * (size_t)n_q * (size_t)(head_dim + 1) * sizeof(float);
@@ -139,6 +180,34 @@ inline int make_prefill_params(const PrefillArgs& a, PrefillParams& p, int64_t& 
   const int64_t rows = (int64_t)a.max_len_extend * p.group;
   const int64_t n_qblk = (rows + block_rows - 1) / block_rows;
   const int64_t n_pairs = a.batch * a.n_kv;
+  p.ragged_tiles = 0;
+  p.ragged_units = 0;
+  p.ragged_rows = 0;
+  p.req_units = nullptr;
+  if (a.ragged_tiles > 0 && n_qblk == 1) {
+    const int64_t units = prefill_ragged_units(a.batch, a.total_kv, a.ragged_tiles);
+    p.n_ksplit = 1;
+    p.ragged_tiles = a.ragged_tiles;
+    p.ragged_units = (int32_t)units;
+    p.ragged_rows = (int32_t)rows;
+    if (!prefill_ragged_never_splits(a.batch, a.total_kv, a.ragged_tiles)) {
+      if (!a.workspace) return MSGL_ERR_WORKSPACE;
+      const int64_t part_rows = units * a.n_kv * rows;
+      p.part_rows = part_rows;
+      p.part_o = static_cast<float*>(a.workspace);
+      p.part_lse = p.part_o + part_rows * a.head_dim;
+      p.req_units = reinterpret_cast<int32_t*>(p.part_lse + part_rows);
+    }
+    n_blocks = units * a.n_kv;
+    if (n_blocks > 0x7fffffffLL) return MSGL_ERR_SHAPE;
+    p.n_qblk = 1;
+    p.n_pairs = (int32_t)n_pairs;
+    p.xcds_per_unit = 1;
+    wide = (uint64_t)a.num_slots * (uint64_t)a.k_stride0 * 2u >= (1ull << 32) ||
+           (uint64_t)a.num_slots * (uint64_t)a.v_stride0 * 2u >= (1ull << 32) ||
+           a.num_slots >= (1 << 24) || a.k_stride0 * 2 >= (1 << 24) || a.v_stride0 * 2 >= (1 << 24);
+    return MSGL_OK;
+  }
   p.xcds_per_unit = prefill_xcds_per_unit(n_pairs * p.n_ksplit);
   n_blocks = 8 * prefill_blocks_per_xcd(n_pairs * p.n_ksplit, n_qblk);
   if (n_qblk <= 0 || n_blocks <= 0) {

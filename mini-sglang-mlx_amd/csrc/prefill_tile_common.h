@@ -89,6 +89,65 @@ __device__ __forceinline__ BlockWork prefill_block_work(const PrefillParams& p) 
   return w;
 }
 
+// ---- ragged shares: which (request, share) is unit `u`? ------------------------------------------
+// Visible key range of a request's only query block (rows 0 .. q_len * group - 1), the floor
+// rounded down to a tile: the kernels compute the same for their block.
+__device__ __forceinline__ void ragged_key_range(const PrefillParams& p, int b, int* k_lo, int* k_hi, int* q_len) {
+  const int ql = min(p.qo_indptr[b + 1] - p.qo_indptr[b], p.max_len_extend);
+  const int kn = max(p.kv_indptr[b + 1] - p.kv_indptr[b], 0);
+  const int prefix = p.prefix_lens[b];
+  int hi = p.is_cross ? kn : min(kn, prefix + ql);
+  int lo = (p.window > 0) ? max(0, prefix - p.window + 1) : 0;
+  lo &= ~(kBN - 1);
+  if (hi < lo) hi = lo;
+  *k_lo = lo;
+  *k_hi = hi;
+  *q_len = ql;
+}
+struct RaggedUnit {
+  int request, share, count, first;  // count = shares of the request, first = its first unit
+  bool ok;                           // false: `u` lies past the last unit
+};
+// Every thread of the workgroup calls it.  A request with rows has at least one share (which
+// writes zeros if it sees no key); a request without rows has none.
+template <int THREADS>
+__device__ __forceinline__ RaggedUnit ragged_unit(const PrefillParams& p, int u, int tid) {
+  __shared__ int count[kRaggedMaxBatch];
+  __shared__ int found[4];
+  if (tid == 0) found[0] = -1;
+  for (int i = tid; i < p.batch; i += THREADS) {
+    int lo, hi, ql;
+    ragged_key_range(p, i, &lo, &hi, &ql);
+    const int tiles = (hi - lo + kBN - 1) / kBN;
+    count[i] = ql > 0 ? max(1, (tiles + p.ragged_tiles - 1) / p.ragged_tiles) : 0;
+  }
+  __syncthreads();
+  if (tid < kWave) {
+    int base = 0;
+    for (int i0 = 0; i0 < p.batch && base <= u; i0 += kWave) {
+      const int i = i0 + tid;
+      const int c = i < p.batch ? count[i] : 0;
+      const int incl = wave_inclusive_scan(c);
+      const int first = base + incl - c;
+      if (c > 0 && u >= first && u < first + c) {
+        found[0] = i;
+        found[1] = u - first;
+        found[2] = c;
+        found[3] = first;
+      }
+      base += __shfl(incl, kWave - 1, kWave);
+    }
+  }
+  __syncthreads();
+  RaggedUnit r;
+  r.request = found[0];
+  r.share = found[1];
+  r.count = found[2];
+  r.first = found[3];
+  r.ok = found[0] >= 0;
+  return r;
+}
+
 typedef int i32x4_t __attribute__((ext_vector_type(4)));
 template <int THREADS>
 __device__ __forceinline__ int request_of_rank(const int32_t* kv_indptr, int batch, int want_rank, int tid) {

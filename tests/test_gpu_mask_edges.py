@@ -34,12 +34,26 @@ def test_decode_sees_every_key_once(gpu, kv_lens):
 
 @pytest.mark.parametrize("is_cross,window", MASKS)
 @pytest.mark.parametrize("q_len", [1, 8, 12, 16])
-def test_split_k_route_mask_edges(gpu, q_len, is_cross, window):
+def test_split_k_route_mask_edges(gpu, tuning, q_len, is_cross, window):
+    from mini_sglang_amd_kernel import _lib
+
+    tuning(_lib.TUNE_SMALLQ_MAXCOLS, 64)  # 64 columns would go to the tile kernel by default
     wl = one_hot_values(build_workload(
         "e", "prefill", seed=6, n_q=16, n_kv=4, kv_lens=[q_len + 3000, q_len + 1023, q_len + 1024, q_len + 7777],
         extend_lens=[q_len] * 4, pool_factor=1.1, is_cross_attention=is_cross,
         sliding_window_size=window))
     _check(wl, gpu, f"split-K q_len={q_len} cross={is_cross} W={window}")
+
+
+@pytest.mark.parametrize("is_cross,window", MASKS)
+@pytest.mark.parametrize("q_len", [16, 50])
+def test_tile_route_ragged_shares_mask_edges(gpu, q_len, is_cross, window):
+    # one query block per (request, kv head) on the tile kernel: requests of 1 to 8 key shares
+    wl = one_hot_values(build_workload(
+        "e", "prefill", seed=8, n_q=16, n_kv=4, kv_lens=[q_len + 9000, q_len + 1023, q_len + 1024, q_len + 4100],
+        extend_lens=[q_len] * 4, pool_factor=1.1, is_cross_attention=is_cross,
+        sliding_window_size=window))
+    _check(wl, gpu, f"tile route, ragged shares q_len={q_len} cross={is_cross} W={window}")
 
 
 @pytest.fixture(params=[0, 1, 3], ids=["pingpong", "4x64rows", "8x32rows"])

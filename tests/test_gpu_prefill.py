@@ -92,9 +92,13 @@ def test_tile_route_group_sizes(gpu, tile_variant, n_q, n_kv):
 
 @pytest.mark.parametrize("is_cross,window", MASKS)
 @pytest.mark.parametrize("q_len", [1, 3, 8, 11, 16])
-def test_splitk_route_masks(gpu, q_len, is_cross, window):
+def test_splitk_route_masks(gpu, tuning, q_len, is_cross, window):
     # short query blocks (verify / draft proposal): q_len * group <= 64; one, two and three
-    # tiles of 16 columns in a wave (q_len 3, 8, 11), four on two waves (16)
+    # tiles of 16 columns in a wave (q_len 3, 8, 11), four on two waves (16: by default these go
+    # to the tile kernel, so the split-K kernel is asked for)
+    from mini_sglang_amd_kernel import _lib
+
+    tuning(_lib.TUNE_SMALLQ_MAXCOLS, 64)
     wl = build_workload("t", "prefill", seed=300 + q_len, n_q=16, n_kv=4,
                         kv_lens=[q_len, 40 + q_len, 333 + q_len, 1500 + q_len],
                         extend_lens=[q_len] * 4, pool_factor=1.3, store_new=True,
@@ -432,3 +436,16 @@ def test_partially_filled_query_blocks_idle_waves(gpu, head_dim):
     _lib.set_tuning(_lib.TUNE_SMALLQ_MAXCOLS, -1)
     _check(wl, gpu, f"partially filled query blocks head_dim={head_dim}")
     _lib.set_tuning(_lib.TUNE_SMALLQ_MAXCOLS, 0)
+
+
+@pytest.mark.parametrize("is_cross,window", MASKS)
+@pytest.mark.parametrize("q_len", [13, 16, 40, 64])
+def test_tile_route_ragged_key_shares(gpu, q_len, is_cross, window):
+    """One query block per (request, kv head) on the tile kernel (49-256 rows at group 4): the
+    keys of a request go in as many equal shares as its length asks for, so one request here has
+    dozens of shares, others one, one has no prefix and one no rows at all."""
+    wl = build_workload("t", "prefill", seed=350 + q_len, n_q=16, n_kv=4,
+                        kv_lens=[q_len + 70000, q_len + 300, q_len + 5000, q_len, 0, q_len + 1300],
+                        extend_lens=[q_len, q_len, q_len, q_len, 0, q_len], pool_factor=1.1,
+                        store_new=True, is_cross_attention=is_cross, sliding_window_size=window)
+    _check(wl, gpu, f"tile route, ragged shares, q_len={q_len} cross={is_cross} W={window}")
