@@ -269,7 +269,8 @@ MSGL_API int msgl_gdn_state_inplace(const void* q, const void* k, const void* v,
  * other threads set.  Read at launch time; not part of the reference surface.
  *   MSGL_TUNE_SEGMENTS       segments the split-K kernel cuts the visible token stream into
  *   MSGL_TUNE_MIN_SEGMENT    smallest segment length in tokens (multiple of 64)
- *   MSGL_TUNE_SMALLQ_MAXCOLS largest q_len*group routed to the split-K kernel
+ *   MSGL_TUNE_SMALLQ_MAXCOLS largest q_len*group routed to the split-K kernel (up to 64; default
+ *                            48 at head_dim 128, 64 at head_dim 256; negative: never)
  *   MSGL_TUNE_PREFILL_VARIANT head_dim 128 MFMA kernel: 0 the ping-pong kernel (8 waves x 32 rows,
  *                            the two waves of a SIMD alternate between MFMA and softmax phases),
  *                            3 the fused kernel it replaced (8 x 32), 1 the fused kernel with
@@ -282,7 +283,9 @@ MSGL_API int msgl_gdn_state_inplace(const void* q, const void* k, const void* v,
  *   MSGL_TUNE_GDN_ROWS       state rows per 16-lane group of the gdn_state kernel: 1, 2, 4
  *                            (0: chosen from the problem size)
  *   MSGL_TUNE_PREFILL_KEY_SPLITS  workgroups that share the keys of one query block of the MFMA
- *                            tile kernels (1: never split, up to 32; 0: chosen from the sizes)
+ *                            tile kernels (1: never split, up to 32; 0: chosen from the sizes,
+ *                            and launches with one query block per request and kv head give each
+ *                            request as many shares as its length asks for)
  */
 #define MSGL_TUNE_SEGMENTS 0
 #define MSGL_TUNE_MIN_SEGMENT 1
