@@ -48,13 +48,13 @@ int32_t segments(int64_t total_kv, int64_t n_kv, int64_t head_dim, int64_t cols)
 // Largest q_len * group that takes the split-K route.  Default at head_dim 128: 48 (up to three
 // column tiles in one wave); 49-64 columns would run on two waves per kv head that each read
 // every K / V row, and the tile kernel with ragged key shares is as fast or faster on them.
-// head_dim 256 keeps every short query block on the split-K kernel (its tile kernel has no
-// ragged shares, and uniform ones make one long request among short ones 4-6 x slower).
+// head_dim 256: 16 (one column tile; more would be a wave per tile, each reading every row,
+// and the tile kernel with ragged shares is 10-65 % faster from 17 columns on).
 int64_t smallq_max_cols(int64_t head_dim) {
   const int64_t t = t_tune[MSGL_TUNE_SMALLQ_MAXCOLS];
   if (t < 0) return 0;  // negative: never take the split-K route
   if (t > 0) return t < msgl::kSplitKvMaxCols ? t : msgl::kSplitKvMaxCols;
-  return head_dim == 128 ? 48 : msgl::kSplitKvMaxCols;
+  return head_dim == 128 ? 48 : 16;
 }
 
 }  // namespace
@@ -223,11 +223,11 @@ int msgl_paged_decode_attention_noalloc(const void* q, const void* k_cache, cons
                           k_cache_stride0, v_cache_stride0, sm_scale, max_kv_splits, dtype, stream);
 }
 
-// Ragged key shares for the tile kernels (one query block per (request, kv head)): head_dim 128
-// with the ping-pong kernel only for now.
+// Ragged key shares for the tile kernels (one query block per (request, kv head)): the ping-pong
+// kernel and the head_dim 256 kernel know them, the fused head_dim 128 kernels do not.
 static int ragged_tiles(int64_t batch, int64_t total_kv, int64_t n_kv, int64_t group,
                         int64_t max_len_extend, int64_t head_dim) {
-  if (head_dim != 128 || msgl::tile_variant() != 0) return 0;
+  if (head_dim == 128 ? msgl::tile_variant() != 0 : msgl::tile_variant() == 2) return 0;
   return msgl::prefill_ragged_tiles(batch, total_kv, n_kv, group, max_len_extend,
                                     msgl::prefill_block_rows(head_dim), t_key_splits);
 }

@@ -71,15 +71,35 @@ __global__ __launch_bounds__(kNW * 64) void prefill_tile256_kernel(PrefillParams
   // XCDs, the q blocks of one (request, kv head, key split) read the same keys, share an XCD and
   // run heaviest first, requests in order of decreasing kv length (each block ranks the requests
   // itself from kv_indptr)
-  const BlockWork work = prefill_block_work(p);
-  if (!work.ok) return;
-  const int unit = work.unit;  // (request, kv head, key split)
-  const int pair = unit / p.n_ksplit;
-  const int split = unit - pair * p.n_ksplit;
-  const int qblk = work.qblk;
-  const int want_rank = pair / p.n_kv;
-  const int kvh = pair - want_rank * p.n_kv;
-  const int b = __builtin_amdgcn_readfirstlane(request_of_rank<kNW * 64>(p.kv_indptr, p.batch, want_rank, tid));
+  // With ragged shares: block -> (unit = (request, share), kv head), see prefill_ragged_tiles().
+  int b, kvh, split, qblk, n_shares = 1;
+  bool to_partial = p.n_ksplit > 1;  // leave a partial for the merge kernel, not the result
+  int64_t part_at = 0;               // partial row of the block's row 0 (ragged shares)
+  if (p.ragged_tiles > 0) {
+    kvh = (int)(blockIdx.x % (unsigned)p.n_kv);
+    const int u = (int)(blockIdx.x / (unsigned)p.n_kv);
+    const RaggedUnit ru = ragged_unit<kNW * 64>(p, u, tid);
+    if (!ru.ok) return;
+    b = __builtin_amdgcn_readfirstlane(ru.request);
+    split = ru.share;
+    qblk = 0;
+    n_shares = ru.count;
+    to_partial = ru.count > 1;
+    part_at = ((int64_t)u * p.n_kv + kvh) * p.ragged_rows;
+    if (ru.share == 0 && kvh == 0 && tid == 0 && p.req_units != nullptr) {
+      p.req_units[2 * b] = ru.first;  // tells the merge kernel where the request's partials are
+      p.req_units[2 * b + 1] = ru.count;
+    }
+  } else {
+    const BlockWork work = prefill_block_work(p);
+    if (!work.ok) return;
+    const int pair = work.unit / p.n_ksplit;  // unit = (request, kv head, key split)
+    split = work.unit - pair * p.n_ksplit;
+    qblk = work.qblk;
+    const int want_rank = pair / p.n_kv;
+    kvh = pair - want_rank * p.n_kv;
+    b = __builtin_amdgcn_readfirstlane(request_of_rank<kNW * 64>(p.kv_indptr, p.batch, want_rank, tid));
+  }
 
   const int q_start = __builtin_amdgcn_readfirstlane(p.qo_indptr[b]);
   const int q_len = min(__builtin_amdgcn_readfirstlane(p.qo_indptr[b + 1]) - q_start, p.max_len_extend);
@@ -98,9 +118,10 @@ __global__ __launch_bounds__(kNW * 64) void prefill_tile256_kernel(PrefillParams
   if (k_hi < k_lo) k_hi = k_lo;
   // key split `split` of n_ksplit: a whole number of step pairs (64 keys) each, the last takes
   // the ragged end; shares past the end are empty (they still leave a "nothing seen" partial)
-  if (p.n_ksplit > 1) {
+  if (p.ragged_tiles > 0 || p.n_ksplit > 1) {
+    const int shares = p.ragged_tiles > 0 ? n_shares : p.n_ksplit;  // ragged: the request's own count
     const int all_pairs = (k_hi - k_lo + 2 * kHalf - 1) / (2 * kHalf);
-    const int share = (all_pairs + p.n_ksplit - 1) / p.n_ksplit * 2 * kHalf;
+    const int share = (all_pairs + shares - 1) / shares * 2 * kHalf;
     k_lo = min(k_lo + split * share, k_hi);
     k_hi = min(k_hi, k_lo + share);
   }
@@ -489,7 +510,7 @@ __global__ __launch_bounds__(kNW * 64) void prefill_tile256_kernel(PrefillParams
   }
 
   // accumulator i of O^T tile dt is dim 32dt + 8(i/4) + 4h + i%4 of query row c32
-  if (p.n_ksplit > 1) {
+  if (to_partial) {
     // ---- key split: normalised fp32 partial and log-sum-exp (base 2) per row, from registers
     float l = l_run;
     l += __shfl_xor(l, 32, kWave);
@@ -498,7 +519,8 @@ __global__ __launch_bounds__(kNW * 64) void prefill_tile256_kernel(PrefillParams
     if (row < rows_total) {
       const int qi = row / p.group;
       const int hh = row - qi * p.group;
-      const int64_t at = (int64_t)split * p.part_rows + (int64_t)(q_start + qi) * p.n_q + kvh * p.group + hh;
+      const int64_t at = p.ragged_tiles > 0 ? part_at + row
+                                            : (int64_t)split * p.part_rows + (int64_t)(q_start + qi) * p.n_q + kvh * p.group + hh;
       if (h == 0) p.part_lse[at] = (l > 0.f) ? m_run + __log2f(l) : kNegInf;
       float* dst = p.part_o + at * kD + 4 * h;
 #pragma unroll
@@ -558,7 +580,7 @@ int launch_prefill_tile256(const PrefillArgs& a, hipStream_t stream) {
   if (wide) hipLaunchKernelGGL((prefill_tile256_kernel<true>), grid, dim3(kNW * 64), 0, stream, p);
   else hipLaunchKernelGGL((prefill_tile256_kernel<false>), grid, dim3(kNW * 64), 0, stream, p);
   const int launched = check_launch();
-  if (launched != MSGL_OK || p.n_ksplit == 1) return launched;
+  if (launched != MSGL_OK || (p.n_ksplit == 1 && p.ragged_tiles == 0)) return launched;
   return launch_prefill_merge(p, kD, stream);
 }
 

@@ -46,11 +46,11 @@ def test_split_k_route_mask_edges(gpu, tuning, q_len, is_cross, window):
 
 
 @pytest.mark.parametrize("is_cross,window", MASKS)
-@pytest.mark.parametrize("q_len", [16, 50])
-def test_tile_route_ragged_shares_mask_edges(gpu, q_len, is_cross, window):
-    # one query block per (request, kv head) on the tile kernel: requests of 1 to 8 key shares
+@pytest.mark.parametrize("head_dim,q_len", [(128, 16), (128, 50), (256, 8), (256, 30)])
+def test_tile_route_ragged_shares_mask_edges(gpu, head_dim, q_len, is_cross, window):
+    # one query block per (request, kv head) on the tile kernels: requests of 1 to 8 key shares
     wl = one_hot_values(build_workload(
-        "e", "prefill", seed=8, n_q=16, n_kv=4, kv_lens=[q_len + 9000, q_len + 1023, q_len + 1024, q_len + 4100],
+        "e", "prefill", seed=8, n_q=16, n_kv=4, head_dim=head_dim, kv_lens=[q_len + 9000, q_len + 1023, q_len + 1024, q_len + 4100],
         extend_lens=[q_len] * 4, pool_factor=1.1, is_cross_attention=is_cross,
         sliding_window_size=window))
     _check(wl, gpu, f"tile route, ragged shares q_len={q_len} cross={is_cross} W={window}")

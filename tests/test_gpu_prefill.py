@@ -197,9 +197,13 @@ def test_head_dim_256_tile_kernel_unusual_scales_and_magnitudes(gpu, scale):
 @pytest.mark.parametrize("head_dim", [128, 256])
 @pytest.mark.parametrize("n_q,n_kv,q_len", [(8, 8, 36), (8, 8, 48), (8, 4, 20), (4, 4, 64), (6, 2, 11),
                                             (8, 8, 17), (16, 1, 3)])
-def test_splitk_route_every_column_tile_count(gpu, head_dim, n_q, n_kv, q_len):
+def test_splitk_route_every_column_tile_count(gpu, tuning, head_dim, n_q, n_kv, q_len):
     # q_len * group = 36, 48, 40, 64, 33, 17, 48 columns: two, three and four tiles of 16, the
-    # three-tile ones with an idle fourth wave per kv head at head_dim 256
+    # three-tile ones with an idle fourth wave per kv head at head_dim 256 (by default most of
+    # these column counts go to the tile kernels, so the split-K kernel is asked for)
+    from mini_sglang_amd_kernel import _lib
+
+    tuning(_lib.TUNE_SMALLQ_MAXCOLS, 64)
     wl = build_workload("t", "prefill", seed=390 + q_len, n_q=n_q, n_kv=n_kv, head_dim=head_dim,
                         kv_lens=[q_len + 32, 500 + q_len, q_len], extend_lens=[q_len] * 3,
                         pool_factor=1.2, store_new=True, sliding_window_size=0)
@@ -439,12 +443,14 @@ def test_partially_filled_query_blocks_idle_waves(gpu, head_dim):
 
 
 @pytest.mark.parametrize("is_cross,window", MASKS)
-@pytest.mark.parametrize("q_len", [13, 16, 40, 64])
-def test_tile_route_ragged_key_shares(gpu, q_len, is_cross, window):
-    """One query block per (request, kv head) on the tile kernel (49-256 rows at group 4): the
-    keys of a request go in as many equal shares as its length asks for, so one request here has
-    dozens of shares, others one, one has no prefix and one no rows at all."""
-    wl = build_workload("t", "prefill", seed=350 + q_len, n_q=16, n_kv=4,
+@pytest.mark.parametrize("head_dim,q_len", [(128, 13), (128, 16), (128, 40), (128, 64), (256, 5),
+                                            (256, 13), (256, 32)])
+def test_tile_route_ragged_key_shares(gpu, head_dim, q_len, is_cross, window):
+    """One query block per (request, kv head) on the tile kernels (52-256 rows at group 4, up to
+    128 at head_dim 256): the keys of a request go in as many equal shares as its length asks
+    for, so one request here has dozens of shares, others one, one has no prefix and one no rows
+    at all."""
+    wl = build_workload("t", "prefill", seed=350 + q_len, n_q=16, n_kv=4, head_dim=head_dim,
                         kv_lens=[q_len + 70000, q_len + 300, q_len + 5000, q_len, 0, q_len + 1300],
                         extend_lens=[q_len, q_len, q_len, q_len, 0, q_len], pool_factor=1.1,
                         store_new=True, is_cross_attention=is_cross, sliding_window_size=window)
