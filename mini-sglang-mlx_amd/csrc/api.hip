@@ -235,6 +235,19 @@ static int ragged_tiles(int64_t batch, int64_t total_kv, int64_t n_kv, int64_t g
 static bool use_splitkv_route(int64_t group, int64_t max_len_extend, int64_t head_dim) {
   return max_len_extend >= 1 && group * max_len_extend <= smallq_max_cols(head_dim);
 }
+// Under a sliding window that most requests exceed (mean kv length at least twice the window),
+// every request shows about `window` keys, the one case where one workgroup per (request, kv
+// head) is balanced: the tile kernel then streams 5-20 % faster than the split-K kernel from
+// 17 columns on (shape 5 with a window of 1024: 32 against 36 us).  Only the default routing
+// does this; MSGL_TUNE_SMALLQ_MAXCOLS set by hand is obeyed as it stands.
+static bool window_prefers_tiles(int64_t batch, int64_t total_kv, int64_t n_kv, int64_t group,
+                                 int64_t max_len_extend, int64_t head_dim, int64_t window) {
+  if (window <= 0 || head_dim != 128 || t_tune[MSGL_TUNE_SMALLQ_MAXCOLS] != 0) return false;
+  if (group * max_len_extend <= 16) return false;
+  if (total_kv < 2 * batch * (window + max_len_extend)) return false;
+  return ragged_tiles(batch, total_kv, n_kv, group, max_len_extend, head_dim) > 0;
+}
+
 // Longer queries run the MFMA tile kernels.  The older route for head_dim 256, the split-K
 // kernel once per chunk of queries (each launch re-reads the visible keys), is kept behind
 // MSGL_TUNE_PREFILL_VARIANT = 2 for comparison.
@@ -268,9 +281,15 @@ size_t msgl_paged_prefill_workspace_bytes(int64_t batch, int64_t total_q, int64_
     return msgl::splitkv_workspace_bytes(batch, num_q_heads, num_kv_heads, head_dim, qc,
                                          segments(total_kv, num_kv_heads, head_dim, group * qc));
   }
-  return msgl::splitkv_workspace_bytes(
+  const size_t split_need = msgl::splitkv_workspace_bytes(
       batch, num_q_heads, num_kv_heads, head_dim, max_len_extend,
       segments(total_kv, num_kv_heads, head_dim, group * max_len_extend));
+  // a sliding window (unknown here) may send the launch to the tile kernel instead
+  const int ragged = ragged_tiles(batch, total_kv, num_kv_heads, group, max_len_extend, head_dim);
+  const size_t tile_need = ragged > 0 ? msgl::prefill_ragged_workspace_bytes(batch, total_kv, num_kv_heads, group,
+                                                                             max_len_extend, head_dim, ragged)
+                                      : 0;
+  return std::max(split_need, tile_need);
 }
 
 int msgl_paged_prefill_attention(const void* q, const void* k_cache, const void* v_cache,
@@ -296,7 +315,9 @@ int msgl_paged_prefill_attention(const void* q, const void* k_cache, const void*
     return MSGL_ERR_NULL_POINTER;
   const int64_t group = num_q_heads / num_kv_heads;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const bool direct = use_splitkv_route(group, max_len_extend, head_dim);
+  const bool direct = use_splitkv_route(group, max_len_extend, head_dim) &&
+                      !window_prefers_tiles(batch, total_kv, num_kv_heads, group, max_len_extend, head_dim,
+                                            sliding_window_size);
   if (direct || use_chunked_route(head_dim, group)) {
     const int32_t per_launch = direct ? max_len_extend : chunk_queries(group);
     const int32_t n_seg = segments(total_kv, num_kv_heads, head_dim, group * per_launch);
