@@ -747,7 +747,11 @@ __global__ __launch_bounds__(512) void prefill_pingpong_kernel(PrefillParams p) 
   const int n_tiles = (k_hi - k_lo + kBN - 1) / kBN;
 
   // ---- this lane's row: Q operand, visibility bounds ---------------------------------------
+  // (the Q rows themselves are requested in the prologue, after the first tiles' slot ids: the
+  // ids gate the first tile moves, and a wait for them would otherwise wait for the Q rows too)
   bf16x8_t qreg[KSTEPS];
+  bool q_valid;
+  int64_t q_off;
   int row_lo, row_hi;
   int w_lo_max = -0x7fffffff, w_hi_min = 0x7fffffff;
   {
@@ -755,13 +759,8 @@ __global__ __launch_bounds__(512) void prefill_pingpong_kernel(PrefillParams p) 
     const bool valid = row < rows_total;
     const int qi = valid ? row / p.group : 0;
     const int hh = valid ? row - qi * p.group : 0;
-    const int64_t off = ((int64_t)(q_start + qi) * p.n_q + kvh * p.group + hh) * D;
-#pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) {
-      u32x4_t raw = {0u, 0u, 0u, 0u};
-      if (valid) raw = ld_global_b128(p.q + off + ks * 16 + h * 8);
-      qreg[ks] = as_bf16x8(raw);
-    }
+    q_valid = valid;
+    q_off = ((int64_t)(q_start + qi) * p.n_q + kvh * p.group + hh) * D;
     const int qpos = prefix + qi;
     int lo = (p.window > 0) ? qpos - p.window + 1 : 0;
     int hi = min(p.is_cross ? kn - 1 : min(qpos, kn - 1), k_hi - 1);
@@ -1062,6 +1061,12 @@ __global__ __launch_bounds__(512) void prefill_pingpong_kernel(PrefillParams p) 
 #pragma unroll
         for (int i = 0; i < UPW; ++i)
           first[t][i] = min((uint32_t)idx_base[min(k_lo + t * kBN + unit_key + i, kn - 1)], p.max_slot);
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ++ks) {
+        u32x4_t raw = {0u, 0u, 0u, 0u};
+        if (q_valid) raw = ld_global_b128(p.q + q_off + ks * 16 + h * 8);
+        qreg[ks] = as_bf16x8(raw);
+      }
       ring_fetch(3);
       ring_fetch(4);
 #pragma unroll
