@@ -270,7 +270,8 @@ MSGL_API int msgl_gdn_state_inplace(const void* q, const void* k, const void* v,
  *   MSGL_TUNE_SEGMENTS       segments the split-K kernel cuts the visible token stream into
  *   MSGL_TUNE_MIN_SEGMENT    smallest segment length in tokens (multiple of 64)
  *   MSGL_TUNE_SMALLQ_MAXCOLS largest q_len*group routed to the split-K kernel (up to 64; default
- *                            48 at head_dim 128, 16 at head_dim 256; negative: never)
+ *                            48 at head_dim 128, 16 at head_dim 256, 64 beyond 128 requests; negative:
+ *                            never)
  *   MSGL_TUNE_PREFILL_VARIANT head_dim 128 MFMA kernel: 0 the ping-pong kernel (8 waves x 32 rows,
  *                            the two waves of a SIMD alternate between MFMA and softmax phases),
  *                            3 the fused kernel it replaced (8 x 32), 1 the fused kernel with

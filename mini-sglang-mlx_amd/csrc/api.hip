@@ -50,10 +50,14 @@ int32_t segments(int64_t total_kv, int64_t n_kv, int64_t head_dim, int64_t cols)
 // every K / V row, and the tile kernel with ragged key shares is as fast or faster on them.
 // head_dim 256: 16 (one column tile; more would be a wave per tile, each reading every row,
 // and the tile kernel with ragged shares is 10-65 % faster from 17 columns on).
-int64_t smallq_max_cols(int64_t head_dim) {
+// With more requests than the tile kernels give ragged shares to (kRaggedMaxBatch), every short
+// query block stays on the split-K kernel: its segments are balanced whatever the lengths, and
+// one long request among many short ones would otherwise be one long workgroup per kv head.
+int64_t smallq_max_cols(int64_t head_dim, int64_t batch) {
   const int64_t t = t_tune[MSGL_TUNE_SMALLQ_MAXCOLS];
   if (t < 0) return 0;  // negative: never take the split-K route
   if (t > 0) return t < msgl::kSplitKvMaxCols ? t : msgl::kSplitKvMaxCols;
+  if (batch > msgl::kRaggedMaxBatch) return msgl::kSplitKvMaxCols;
   return head_dim == 128 ? 48 : 16;
 }
 
@@ -232,8 +236,8 @@ static int ragged_tiles(int64_t batch, int64_t total_kv, int64_t n_kv, int64_t g
                                     msgl::prefill_block_rows(head_dim), t_key_splits);
 }
 
-static bool use_splitkv_route(int64_t group, int64_t max_len_extend, int64_t head_dim) {
-  return max_len_extend >= 1 && group * max_len_extend <= smallq_max_cols(head_dim);
+static bool use_splitkv_route(int64_t group, int64_t max_len_extend, int64_t head_dim, int64_t batch) {
+  return max_len_extend >= 1 && group * max_len_extend <= smallq_max_cols(head_dim, batch);
 }
 // Under a sliding window that most requests exceed (mean kv length at least twice the window),
 // every request shows about `window` keys, the one case where one workgroup per (request, kv
@@ -255,7 +259,7 @@ static bool use_chunked_route(int64_t head_dim, int64_t group) {
   return head_dim == 256 && msgl::tile_variant() == 2 && group <= msgl::kSplitKvMaxCols;
 }
 static int32_t chunk_queries(int64_t group) {
-  return (int32_t)std::max<int64_t>(1, std::min<int64_t>(smallq_max_cols(256), msgl::kSplitKvMaxCols) / group);
+  return (int32_t)std::max<int64_t>(1, std::min<int64_t>(smallq_max_cols(256, 1 << 30), msgl::kSplitKvMaxCols) / group);
 }
 
 size_t msgl_paged_prefill_workspace_bytes(int64_t batch, int64_t total_q, int64_t total_kv,
@@ -265,7 +269,7 @@ size_t msgl_paged_prefill_workspace_bytes(int64_t batch, int64_t total_q, int64_
       num_q_heads % num_kv_heads != 0)
     return 0;
   const int64_t group = num_q_heads / num_kv_heads;
-  if (!use_splitkv_route(group, max_len_extend, head_dim)) {
+  if (!use_splitkv_route(group, max_len_extend, head_dim, batch)) {
     if (!use_chunked_route(head_dim, group)) {
       // tile kernels: partials of a key split, if this launch would use one (a sliding window,
       // unknown here, can only lower the count)
@@ -315,7 +319,7 @@ int msgl_paged_prefill_attention(const void* q, const void* k_cache, const void*
     return MSGL_ERR_NULL_POINTER;
   const int64_t group = num_q_heads / num_kv_heads;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const bool direct = use_splitkv_route(group, max_len_extend, head_dim) &&
+  const bool direct = use_splitkv_route(group, max_len_extend, head_dim, batch) &&
                       !window_prefers_tiles(batch, total_kv, num_kv_heads, group, max_len_extend, head_dim,
                                             sliding_window_size);
   if (direct || use_chunked_route(head_dim, group)) {
