@@ -56,11 +56,6 @@ __device__ __forceinline__ u32x2_t lds_read_tr16(const unsigned char* p) {
   return __builtin_bit_cast(u32x2_t, v);
 }
 
-// The request whose kv length has rank `want_rank` in decreasing order (ties: lower index first),
-// found by the workgroup itself: lengths into LDS once, then each thread ranks one request
-// against all of them with broadcast LDS reads.  (Ranking straight from global memory cost every
-// workgroup of a 64-request launch 3.4 us.)  Every thread of the workgroup calls it; beyond
-// kRankedBatch requests the order is the batch order.
 // Workgroup id -> (unit = (request rank, kv head, key split), query block), heaviest query block
 // (latest rows) first; `ok` is false for the ids that pad the grid.  Consecutive ids go to
 // different XCDs.
@@ -148,6 +143,11 @@ __device__ __forceinline__ RaggedUnit ragged_unit(const PrefillParams& p, int u,
   return r;
 }
 
+// The request whose kv length has rank `want_rank` in decreasing order (ties: lower index first),
+// found by the workgroup itself: lengths into LDS once, then each thread ranks one request
+// against all of them with broadcast LDS reads.  (Ranking straight from global memory cost every
+// workgroup of a 64-request launch 3.4 us.)  Every thread of the workgroup calls it; beyond
+// kRankedBatch requests the order is the batch order.
 typedef int i32x4_t __attribute__((ext_vector_type(4)));
 template <int THREADS>
 __device__ __forceinline__ int request_of_rank(const int32_t* kv_indptr, int batch, int want_rank, int tid) {
