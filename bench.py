@@ -730,6 +730,9 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-extra-shapes", action="store_true",
+                    help="skip the legs on shapes outside the benchmark set (small launches, few long "
+                         "requests, the reference's micro-benchmark shapes)")
     ap.add_argument("--configs", default="2,3,1,5,5w,4,3h")
     ap.add_argument("--no-check", action="store_true", help="skip the oracle comparison")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -859,9 +862,10 @@ def main():
         result["radix_prefix_cache"] = run_radix_cache(not args.no_cpu_baseline)
         result["decode_step_graph"] = run_decode_step_graph(dev, args.steps, args.warmup)
         result["state_pool_copy"] = run_state_pool(dev, args.steps, args.warmup, not args.no_cpu_baseline)
-        result["small_launch_extends"] = run_small_launch_extends(dev, args.steps, args.warmup)
-        result["few_long_requests_decode"] = run_few_long_requests_decode(dev, args.steps, args.warmup)
-        result["reference_microbench_shapes"] = run_reference_microbench_shapes(dev, args.steps, args.warmup)
+        if not args.no_extra_shapes:
+            result["small_launch_extends"] = run_small_launch_extends(dev, args.steps, args.warmup)
+            result["few_long_requests_decode"] = run_few_long_requests_decode(dev, args.steps, args.warmup)
+            result["reference_microbench_shapes"] = run_reference_microbench_shapes(dev, args.steps, args.warmup)
     result["all_configs"] = rows
     print(json.dumps(result))
 
