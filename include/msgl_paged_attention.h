@@ -268,7 +268,8 @@ MSGL_API int msgl_gdn_state_inplace(const void* q, const void* k, const void* v,
  * *_workspace_bytes() call and the launch that follows it on the same thread agree whatever
  * other threads set.  Read at launch time; not part of the reference surface.
  *   MSGL_TUNE_SEGMENTS       segments the split-K kernel cuts the visible token stream into
- *   MSGL_TUNE_MIN_SEGMENT    smallest segment length in tokens (multiple of 64)
+ *   MSGL_TUNE_MIN_SEGMENT    smallest segment length in tokens (multiple of 64; default 128 at
+ *                            head_dim 128, 64 at head_dim 256)
  *   MSGL_TUNE_SMALLQ_MAXCOLS largest q_len*group routed to the split-K kernel (up to 64; default
  *                            48 at head_dim 128, 16 at head_dim 256, 64 beyond 128 requests; negative:
  *                            never)

@@ -35,15 +35,18 @@ int check_common(const void* q, const void* k_cache, const void* v_cache, const 
   return MSGL_OK;
 }
 
-int32_t min_segment() {
+// Smallest segment: 128 tokens at head_dim 128 (64 changes nothing there), 64 at head_dim 256,
+// where a workgroup takes twice as long per token and small launches gain 15-20 % from the
+// finer cut.
+int32_t min_segment(int64_t head_dim) {
   const int64_t t = t_tune[MSGL_TUNE_MIN_SEGMENT];
   if (t >= 64) return (int32_t)(t / 64 * 64);
-  return msgl::kSplitKvMinSegment;
+  return head_dim == 256 ? 64 : msgl::kSplitKvMinSegment;
 }
 int32_t segments(int64_t total_kv, int64_t n_kv, int64_t head_dim, int64_t cols) {
   const int64_t t = t_tune[MSGL_TUNE_SEGMENTS];
   if (t >= 1) return (int32_t)(t < (1 << 20) ? t : (1 << 20));
-  return msgl::splitkv_default_segments(total_kv, n_kv, head_dim, cols, min_segment());
+  return msgl::splitkv_default_segments(total_kv, n_kv, head_dim, cols, min_segment(head_dim));
 }
 // Largest q_len * group that takes the split-K route.  Default at head_dim 128: 48 (up to three
 // column tiles in one wave); 49-64 columns would run on two waves per kv head that each read
@@ -196,7 +199,7 @@ static int decode_attention(const void* q, const void* k_cache, const void* v_ca
   a.is_cross = 0;
   a.window = 0;
   a.n_seg = n_seg;
-  a.min_seg = min_segment();
+  a.min_seg = min_segment(head_dim);
   return msgl::launch_splitkv(a, static_cast<hipStream_t>(stream));
 }
 
@@ -352,7 +355,7 @@ int msgl_paged_prefill_attention(const void* q, const void* k_cache, const void*
     a.is_cross = is_cross_attention ? 1 : 0;
     a.window = sliding_window_size;
     a.n_seg = n_seg;
-    a.min_seg = min_segment();
+    a.min_seg = min_segment(head_dim);
     // launches share the workspace: they run one after the other on the stream
     for (int32_t q0 = 0; q0 < max_len_extend; q0 += per_launch) {
       a.q_begin = q0;
