@@ -271,8 +271,8 @@ MSGL_API int msgl_gdn_state_inplace(const void* q, const void* k, const void* v,
  *   MSGL_TUNE_MIN_SEGMENT    smallest segment length in tokens (multiple of 64; default 128 at
  *                            head_dim 128, 64 at head_dim 256)
  *   MSGL_TUNE_SMALLQ_MAXCOLS largest q_len*group routed to the split-K kernel (up to 64; default
- *                            48 at head_dim 128, 16 at head_dim 256, 64 beyond 128 requests; negative:
- *                            never)
+ *                            48 at head_dim 128, 16 at head_dim 256, and up to 64 where the tile
+ *                            kernels cannot split a request's keys by its length; negative: never)
  *   MSGL_TUNE_PREFILL_VARIANT head_dim 128 MFMA kernel: 0 the ping-pong kernel (8 waves x 32 rows,
  *                            the two waves of a SIMD alternate between MFMA and softmax phases),
  *                            3 the fused kernel it replaced (8 x 32), 1 the fused kernel with
@@ -287,7 +287,8 @@ MSGL_API int msgl_gdn_state_inplace(const void* q, const void* k, const void* v,
  *   MSGL_TUNE_PREFILL_KEY_SPLITS  workgroups that share the keys of one query block of the MFMA
  *                            tile kernels (1: never split, up to 32; 0: chosen from the sizes,
  *                            and launches with one query block per request and kv head give each
- *                            request as many shares as its length asks for)
+ *                            request as many shares as its length asks for, up to 128 requests
+ *                            or 1024 long ones)
  */
 #define MSGL_TUNE_SEGMENTS 0
 #define MSGL_TUNE_MIN_SEGMENT 1

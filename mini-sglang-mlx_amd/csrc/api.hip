@@ -48,21 +48,15 @@ int32_t segments(int64_t total_kv, int64_t n_kv, int64_t head_dim, int64_t cols)
   if (t >= 1) return (int32_t)(t < (1 << 20) ? t : (1 << 20));
   return msgl::splitkv_default_segments(total_kv, n_kv, head_dim, cols, min_segment(head_dim));
 }
-// Largest q_len * group that takes the split-K route.  Default at head_dim 128: 48 (up to three
-// column tiles in one wave); 49-64 columns would run on two waves per kv head that each read
-// every K / V row, and the tile kernel with ragged key shares is as fast or faster on them.
-// head_dim 256: 16 (one column tile; more would be a wave per tile, each reading every row,
-// and the tile kernel with ragged shares is 10-65 % faster from 17 columns on).
-// With more requests than the tile kernels give ragged shares to (kRaggedMaxBatch), every short
-// query block stays on the split-K kernel: its segments are balanced whatever the lengths, and
-// one long request among many short ones would otherwise be one long workgroup per kv head.
-int64_t smallq_max_cols(int64_t head_dim, int64_t batch) {
-  const int64_t t = t_tune[MSGL_TUNE_SMALLQ_MAXCOLS];
-  if (t < 0) return 0;  // negative: never take the split-K route
-  if (t > 0) return t < msgl::kSplitKvMaxCols ? t : msgl::kSplitKvMaxCols;
-  if (batch > msgl::kRaggedMaxBatch) return msgl::kSplitKvMaxCols;
-  return head_dim == 128 ? 48 : 16;
-}
+// Largest q_len * group that takes the split-K route whatever the launch: at head_dim 128 48 (up
+// to three column tiles in one wave; 49-64 columns would run on two waves per kv head that each
+// read every K / V row, and the tile kernel with ragged key shares is as fast or faster on them),
+// at head_dim 256 16 (one column tile; more would be a wave per tile, each reading every row,
+// and the tile kernel with ragged shares is 10-65 % faster from 17 columns on).  Up to 64 columns
+// the split-K kernel also takes what the tile kernels cannot give ragged shares to (very many
+// or many short requests): its segments are balanced whatever the lengths, and one long request
+// among many short ones would otherwise be one long workgroup per kv head.
+int64_t smallq_base_cols(int64_t head_dim) { return head_dim == 128 ? 48 : 16; }
 
 }  // namespace
 
@@ -239,8 +233,14 @@ static int ragged_tiles(int64_t batch, int64_t total_kv, int64_t n_kv, int64_t g
                                     msgl::prefill_block_rows(head_dim), t_key_splits);
 }
 
-static bool use_splitkv_route(int64_t group, int64_t max_len_extend, int64_t head_dim, int64_t batch) {
-  return max_len_extend >= 1 && group * max_len_extend <= smallq_max_cols(head_dim, batch);
+static bool use_splitkv_route(int64_t group, int64_t max_len_extend, int64_t head_dim, int64_t batch,
+                              int64_t total_kv, int64_t n_kv) {
+  const int64_t cols = group * max_len_extend;
+  if (max_len_extend < 1 || cols > msgl::kSplitKvMaxCols) return false;
+  const int64_t t = t_tune[MSGL_TUNE_SMALLQ_MAXCOLS];
+  if (t != 0) return t > 0 && cols <= t;  // set by hand; negative: never
+  if (cols <= smallq_base_cols(head_dim)) return true;
+  return ragged_tiles(batch, total_kv, n_kv, group, max_len_extend, head_dim) == 0;
 }
 // Under a sliding window that most requests exceed (mean kv length at least twice the window),
 // every request shows about `window` keys, the one case where one workgroup per (request, kv
@@ -262,7 +262,7 @@ static bool use_chunked_route(int64_t head_dim, int64_t group) {
   return head_dim == 256 && msgl::tile_variant() == 2 && group <= msgl::kSplitKvMaxCols;
 }
 static int32_t chunk_queries(int64_t group) {
-  return (int32_t)std::max<int64_t>(1, std::min<int64_t>(smallq_max_cols(256, 1 << 30), msgl::kSplitKvMaxCols) / group);
+  return (int32_t)std::max<int64_t>(1, (t_tune[MSGL_TUNE_SMALLQ_MAXCOLS] > 0 ? std::min<int64_t>(t_tune[MSGL_TUNE_SMALLQ_MAXCOLS], msgl::kSplitKvMaxCols) : msgl::kSplitKvMaxCols) / group);
 }
 
 size_t msgl_paged_prefill_workspace_bytes(int64_t batch, int64_t total_q, int64_t total_kv,
@@ -272,7 +272,7 @@ size_t msgl_paged_prefill_workspace_bytes(int64_t batch, int64_t total_q, int64_
       num_q_heads % num_kv_heads != 0)
     return 0;
   const int64_t group = num_q_heads / num_kv_heads;
-  if (!use_splitkv_route(group, max_len_extend, head_dim, batch)) {
+  if (!use_splitkv_route(group, max_len_extend, head_dim, batch, total_kv, num_kv_heads)) {
     if (!use_chunked_route(head_dim, group)) {
       // tile kernels: partials of a key split, if this launch would use one (a sliding window,
       // unknown here, can only lower the count)
@@ -322,7 +322,7 @@ int msgl_paged_prefill_attention(const void* q, const void* k_cache, const void*
     return MSGL_ERR_NULL_POINTER;
   const int64_t group = num_q_heads / num_kv_heads;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const bool direct = use_splitkv_route(group, max_len_extend, head_dim, batch) &&
+  const bool direct = use_splitkv_route(group, max_len_extend, head_dim, batch, total_kv, num_kv_heads) &&
                       !window_prefers_tiles(batch, total_kv, num_kv_heads, group, max_len_extend, head_dim,
                                             sliding_window_size);
   if (direct || use_chunked_route(head_dim, group)) {

@@ -107,8 +107,12 @@ struct RaggedUnit {
 // writes zeros if it sees no key); a request without rows has none.
 template <int THREADS>
 __device__ __forceinline__ RaggedUnit ragged_unit(const PrefillParams& p, int u, int tid) {
+  constexpr int kChunks = kRaggedMaxBatch / kWave;
   __shared__ int count[kRaggedMaxBatch];
+  __shared__ int chunk_sum[kChunks];  // shares of requests 64 c .. 64 c + 63
   __shared__ int found[4];
+  const int lane = tid & (kWave - 1);
+  const int wave = tid / kWave;
   if (tid == 0) found[0] = -1;
   for (int i = tid; i < p.batch; i += THREADS) {
     int lo, hi, ql;
@@ -117,20 +121,30 @@ __device__ __forceinline__ RaggedUnit ragged_unit(const PrefillParams& p, int u,
     count[i] = ql > 0 ? max(1, (tiles + p.ragged_tiles - 1) / p.ragged_tiles) : 0;
   }
   __syncthreads();
-  if (tid < kWave) {
-    int base = 0;
-    for (int i0 = 0; i0 < p.batch && base <= u; i0 += kWave) {
-      const int i = i0 + tid;
-      const int c = i < p.batch ? count[i] : 0;
-      const int incl = wave_inclusive_scan(c);
-      const int first = base + incl - c;
-      if (c > 0 && u >= first && u < first + c) {
-        found[0] = i;
-        found[1] = u - first;
-        found[2] = c;
-        found[3] = first;
-      }
-      base += __shfl(incl, kWave - 1, kWave);
+  const int n_chunks = (p.batch + kWave - 1) / kWave;
+  for (int c = wave; c < n_chunks; c += THREADS / kWave) {
+    const int i = c * kWave + lane;
+    int v = i < p.batch ? count[i] : 0;
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) v += __shfl_xor(v, off, kWave);
+    if (lane == 0) chunk_sum[c] = v;
+  }
+  __syncthreads();
+  int base = 0, c = 0;  // the chunk that holds unit u: the same for every thread
+  for (; c < n_chunks; ++c) {
+    const int sum = chunk_sum[c];
+    if (u < base + sum) break;
+    base += sum;
+  }
+  if (c < n_chunks && wave == 0) {
+    const int i = c * kWave + lane;
+    const int v = i < p.batch ? count[i] : 0;
+    const int first = base + wave_inclusive_scan(v) - v;
+    if (v > 0 && u >= first && u < first + v) {
+      found[0] = i;
+      found[1] = u - first;
+      found[2] = v;
+      found[3] = first;
     }
   }
   __syncthreads();
