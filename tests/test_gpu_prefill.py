@@ -455,3 +455,16 @@ def test_tile_route_ragged_key_shares(gpu, head_dim, q_len, is_cross, window):
                         extend_lens=[q_len, q_len, q_len, q_len, 0, q_len], pool_factor=1.1,
                         store_new=True, is_cross_attention=is_cross, sliding_window_size=window)
     _check(wl, gpu, f"tile route, ragged shares, q_len={q_len} cross={is_cross} W={window}")
+
+
+@pytest.mark.parametrize("head_dim,q_len", [(128, 16), (128, 50), (256, 8)])
+def test_tile_route_ragged_shares_many_requests(gpu, head_dim, q_len):
+    """More than 128 requests keep ragged key shares when they are long on average: 150 requests,
+    one of them twenty times the others, so its shares are spread over three 64-request chunks of
+    the share-count scan; and the same batch with short requests, which the tile kernels take
+    without shares (or, for the short query blocks, the split-K kernel)."""
+    for lens in ([20000] + [1100] * 149, [1100] * 70 + [20000] + [1100] * 79, [3000] + [90] * 149):
+        wl = build_workload("t", "prefill", seed=370 + q_len, n_q=16, n_kv=4, head_dim=head_dim,
+                            kv_lens=[n + q_len for n in lens], extend_lens=[q_len] * len(lens),
+                            pool_factor=1.1, store_new=True)
+        _check(wl, gpu, f"tile route, {len(lens)} requests, d={head_dim} q_len={q_len} first={lens[0]}")
