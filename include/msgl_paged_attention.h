@@ -275,8 +275,8 @@ MSGL_API int msgl_gdn_state_inplace(const void* q, const void* k, const void* v,
  *                            kernels cannot split a request's keys by its length; negative: never)
  *   MSGL_TUNE_PREFILL_VARIANT head_dim 128 MFMA kernel: 0 the ping-pong kernel (8 waves x 32 rows,
  *                            the two waves of a SIMD alternate between MFMA and softmax phases),
- *                            3 the fused kernel it replaced (8 x 32), 1 the fused kernel with
- *                            4 waves x 64 rows; 2: head_dim 256 through split-K in query chunks
+ *                            1 the fused kernel it replaced (8 x 32 rows, every wave a software-
+ *                            pipelined mix of MFMA and softmax), kept as its comparison partner
  *   MSGL_TUNE_SPLITKV_WAVES  most waves (adjacent kv heads) per split-K workgroup: 1, 2, 4, 8
  *                            (0 restores the default, 4)
  *   MSGL_TUNE_SPLITKV_BOUNDARY tokens' worth of time a split-K workgroup is charged for starting

@@ -228,7 +228,7 @@ int msgl_paged_decode_attention_noalloc(const void* q, const void* k_cache, cons
 // kernel and the head_dim 256 kernel know them, the fused head_dim 128 kernels do not.
 static int ragged_tiles(int64_t batch, int64_t total_kv, int64_t n_kv, int64_t group,
                         int64_t max_len_extend, int64_t head_dim) {
-  if (head_dim == 128 ? msgl::tile_variant() != 0 : msgl::tile_variant() == 2) return 0;
+  if (head_dim == 128 && msgl::tile_variant() != 0) return 0;
   return msgl::prefill_ragged_tiles(batch, total_kv, n_kv, group, max_len_extend,
                                     msgl::prefill_block_rows(head_dim), t_key_splits);
 }
@@ -255,16 +255,6 @@ static bool window_prefers_tiles(int64_t batch, int64_t total_kv, int64_t n_kv, 
   return ragged_tiles(batch, total_kv, n_kv, group, max_len_extend, head_dim) > 0;
 }
 
-// Longer queries run the MFMA tile kernels.  The older route for head_dim 256, the split-K
-// kernel once per chunk of queries (each launch re-reads the visible keys), is kept behind
-// MSGL_TUNE_PREFILL_VARIANT = 2 for comparison.
-static bool use_chunked_route(int64_t head_dim, int64_t group) {
-  return head_dim == 256 && msgl::tile_variant() == 2 && group <= msgl::kSplitKvMaxCols;
-}
-static int32_t chunk_queries(int64_t group) {
-  return (int32_t)std::max<int64_t>(1, (t_tune[MSGL_TUNE_SMALLQ_MAXCOLS] > 0 ? std::min<int64_t>(t_tune[MSGL_TUNE_SMALLQ_MAXCOLS], msgl::kSplitKvMaxCols) : msgl::kSplitKvMaxCols) / group);
-}
-
 size_t msgl_paged_prefill_workspace_bytes(int64_t batch, int64_t total_q, int64_t total_kv,
                                           int64_t num_q_heads, int64_t num_kv_heads,
                                           int64_t head_dim, int64_t max_len_extend) {
@@ -273,20 +263,15 @@ size_t msgl_paged_prefill_workspace_bytes(int64_t batch, int64_t total_q, int64_
     return 0;
   const int64_t group = num_q_heads / num_kv_heads;
   if (!use_splitkv_route(group, max_len_extend, head_dim, batch, total_kv, num_kv_heads)) {
-    if (!use_chunked_route(head_dim, group)) {
-      // tile kernels: partials of a key split, if this launch would use one (a sliding window,
-      // unknown here, can only lower the count)
-      const int ragged = ragged_tiles(batch, total_kv, num_kv_heads, group, max_len_extend, head_dim);
-      if (ragged > 0)
-        return msgl::prefill_ragged_workspace_bytes(batch, total_kv, num_kv_heads, group,
-                                                    max_len_extend, head_dim, ragged);
-      const int k = msgl::prefill_key_splits(batch, total_kv, num_kv_heads, group, max_len_extend, 0,
-                                             msgl::prefill_block_rows(head_dim), t_key_splits);
-      return msgl::prefill_split_workspace_bytes(total_q, num_q_heads, head_dim, k);
-    }
-    const int32_t qc = chunk_queries(group);
-    return msgl::splitkv_workspace_bytes(batch, num_q_heads, num_kv_heads, head_dim, qc,
-                                         segments(total_kv, num_kv_heads, head_dim, group * qc));
+    // tile kernels: partials of a key split, if this launch would use one (a sliding window,
+    // unknown here, can only lower the count)
+    const int ragged = ragged_tiles(batch, total_kv, num_kv_heads, group, max_len_extend, head_dim);
+    if (ragged > 0)
+      return msgl::prefill_ragged_workspace_bytes(batch, total_kv, num_kv_heads, group,
+                                                  max_len_extend, head_dim, ragged);
+    const int k = msgl::prefill_key_splits(batch, total_kv, num_kv_heads, group, max_len_extend, 0,
+                                           msgl::prefill_block_rows(head_dim), t_key_splits);
+    return msgl::prefill_split_workspace_bytes(total_q, num_q_heads, head_dim, k);
   }
   const size_t split_need = msgl::splitkv_workspace_bytes(
       batch, num_q_heads, num_kv_heads, head_dim, max_len_extend,
@@ -325,11 +310,10 @@ int msgl_paged_prefill_attention(const void* q, const void* k_cache, const void*
   const bool direct = use_splitkv_route(group, max_len_extend, head_dim, batch, total_kv, num_kv_heads) &&
                       !window_prefers_tiles(batch, total_kv, num_kv_heads, group, max_len_extend, head_dim,
                                             sliding_window_size);
-  if (direct || use_chunked_route(head_dim, group)) {
-    const int32_t per_launch = direct ? max_len_extend : chunk_queries(group);
-    const int32_t n_seg = segments(total_kv, num_kv_heads, head_dim, group * per_launch);
+  if (direct) {
+    const int32_t n_seg = segments(total_kv, num_kv_heads, head_dim, group * max_len_extend);
     const size_t need = msgl::splitkv_workspace_bytes(batch, num_q_heads, num_kv_heads, head_dim,
-                                                      per_launch, n_seg);
+                                                      max_len_extend, n_seg);
     if (!workspace || workspace_bytes < need || !aligned16(workspace)) return MSGL_ERR_WORKSPACE;
     msgl::SplitKvArgs a{};
     a.q = q;
@@ -350,19 +334,14 @@ int msgl_paged_prefill_attention(const void* q, const void* k_cache, const void*
     a.k_stride0 = k_cache_stride0;
     a.v_stride0 = v_cache_stride0;
     a.sm_scale = sm_scale;
-    a.max_len_extend = per_launch;
+    a.max_len_extend = max_len_extend;
     a.q_cap = max_len_extend;
     a.is_cross = is_cross_attention ? 1 : 0;
     a.window = sliding_window_size;
     a.n_seg = n_seg;
     a.min_seg = min_segment(head_dim);
-    // launches share the workspace: they run one after the other on the stream
-    for (int32_t q0 = 0; q0 < max_len_extend; q0 += per_launch) {
-      a.q_begin = q0;
-      rc = msgl::launch_splitkv(a, s);
-      if (rc != MSGL_OK) return rc;
-    }
-    return MSGL_OK;
+    a.q_begin = 0;
+    return msgl::launch_splitkv(a, s);
   }
   msgl::PrefillArgs a{};
   a.q = q;

@@ -985,45 +985,11 @@ __global__ __launch_bounds__(512) void prefill_pingpong_kernel(PrefillParams p) 
   using No = std::false_type;
 
   const bool general_scale = p.scale_log2e <= 0.f;  // the fast path needs a positive scale
-  // V phase j: P(j+1) from S(j+1), then the first operands of M phase j+1
-  auto v_phase = [&](int j, bf16x8_t (&o)[pp::kOperandBuffers][4]) {
-    const int base = k_lo + (j + 1) * kBN;
-    float mul = p.scale_log2e;
-    if (general_scale || base < w_lo_max || base + kBN - 1 > w_hi_min) {
-      // boundary tile: scale and mask in place.  The empty volatile statement keeps this a
-      // branch: as selects it would put 100 more VALU instructions into every tile.
-      asm volatile("" ::: "memory");
-#pragma unroll
-      for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const int key = base + 32 * kt + 8 * (i >> 2) + 4 * h + (i & 3);
-          const float x = s[kt][i] * p.scale_log2e;
-          s[kt][i] = (key < row_lo || key > row_hi) ? kNegInf : x;
-        }
-      mul = 1.0f;
-    }
-    const float mx = fmaxf(half_max(0), half_max(1));
-    float m_safe = m_safe_run, alpha = 1.0f;
-    // Usual case: no lane of the wave saw a score more than kLazy above its row's running max,
-    // so no row's max moves (both halves of a row sit in this wave).  Otherwise the cross-lane
-    // exchange, the new state and, where a max did move, the rescaling of O.
-    if (__any(mx * mul > m_run + kLazy)) {
-      const float m = wave_max_xor(mx * mul, 32);
-      const float m_old = m_run;
-      const float m_new = fmaxf(m_old, m);
-      const float m_use = (m_new - m_old > kLazy) ? m_new : m_old;
-      m_safe = (m_use == kNegInf) ? 0.f : m_use;
-      m_safe_run = m_safe;
-      alpha = fast_exp2(m_old - m_safe);
-      m_run = m_use;
-      if (__any(alpha != 1.0f)) {
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) oacc[dt][i] *= alpha;
-      }
-    }
+  // P of one tile from its scores: exp2(s * mul - m_safe), cut to bf16 (the upper halves of two
+  // fp32 values side by side, one v_perm_b32: truncation; the row sum below is taken from the
+  // same cut values, so the half step they all lose on average cancels in O / l, and what is
+  // left is an error as wide as that of rounding to nearest).  Returns the lane's sum of them.
+  auto exp_pack = [&](float mul, float m_safe) {
     float psum[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int kt = 0; kt < 2; ++kt)
@@ -1034,22 +1000,63 @@ __global__ __launch_bounds__(512) void prefill_pingpong_kernel(PrefillParams p) 
         for (int e = 0; e < 4; ++e) {
           const float e0 = fast_exp2(__builtin_fmaf(s[kt][8 * u + 2 * e], mul, -m_safe));
           const float e1 = fast_exp2(__builtin_fmaf(s[kt][8 * u + 2 * e + 1], mul, -m_safe));
-          const uint32_t pw = pack_bf16x2(e0, e1);
+          const uint32_t pw = pack_hi16(__builtin_bit_cast(uint32_t, e0), __builtin_bit_cast(uint32_t, e1));
           pk[e] = pw;
-          // row sum of the rounded weights, the ones that multiply V
           psum[e] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, pw), kOnes, psum[e], false);
         }
         pb[kt][u] = as_bf16x8(pk);
       }
-    l_run = l_run * alpha + ((psum[0] + psum[1]) + (psum[2] + psum[3]));
+    return (psum[0] + psum[1]) + (psum[2] + psum[3]);
+  };
+  // V phase j: P(j+1) from S(j+1), then the first operands of M phase j+1
+  auto v_phase = [&](int j, bf16x8_t (&o)[pp::kOperandBuffers][4]) {
+    // First of all the operands of the first slice of M phase j+1 (its scores', if it computes
+    // any) are requested: they arrive while the VALU works, and that phase's first MFMA finds
+    // them there.  (The last phase, P V only, asks for its operands itself: the V tile it reads
+    // may only have been published by the barrier that precedes it.)
+    if (j + 2 < n_tiles) k_ops(smem + k_stage_of(j + 2) + k_lane, 0, 0, o[0]);
     __builtin_amdgcn_sched_barrier(0);
-    // operands of the first slice(s) of M phase j+1: its scores' if it computes any, else
-    // its P V's
-    if (j + 2 < n_tiles) {
-      k_ops(smem + k_stage_of(j + 2) + k_lane, 0, 0, o[0]);
+    const int base = k_lo + (j + 1) * kBN;
+    const bool boundary = general_scale || base < w_lo_max || base + kBN - 1 > w_hi_min;
+    {
+      float mul = p.scale_log2e;
+      if (boundary) {
+        // boundary tile: scale and mask in place.  The empty volatile statement keeps this a
+        // branch: as selects it would put 100 more VALU instructions into every tile.
+        asm volatile("" ::: "memory");
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            const int key = base + 32 * kt + 8 * (i >> 2) + 4 * h + (i & 3);
+            const float x = s[kt][i] * p.scale_log2e;
+            s[kt][i] = (key < row_lo || key > row_hi) ? kNegInf : x;
+          }
+        mul = 1.0f;
+      }
+      const float mx = fmaxf(half_max(0), half_max(1));
+      float m_safe = m_safe_run, alpha = 1.0f;
+      // Has some lane seen a score more than kLazy above its row's reference?  If not, no row's
+      // reference moves (both halves of a row sit in this wave).  Otherwise the cross-lane
+      // exchange, the new state and, where a reference did move, the rescaling of O.
+      if (__any(mx * mul > m_run + kLazy)) {
+        const float m = wave_max_xor(mx * mul, 32);
+        const float m_old = m_run;
+        const float m_new = fmaxf(m_old, m);
+        const float m_use = (m_new - m_old > kLazy) ? m_new : m_old;
+        m_safe = (m_use == kNegInf) ? 0.f : m_use;
+        m_safe_run = m_safe;
+        alpha = fast_exp2(m_old - m_safe);
+        m_run = m_use;
+        if (__any(alpha != 1.0f)) {
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) oacc[dt][i] *= alpha;
+        }
+      }
+      l_run = l_run * alpha + exp_pack(mul, m_safe);
     }
-    // (the last phase, P V only, asks for its operands itself: the V tile it reads may only have
-    // been published by the barrier that precedes it)
   };
 
   if (n_tiles > 0) {
@@ -1288,7 +1295,8 @@ int launch_prefill_merge(const PrefillParams& p, int head_dim, hipStream_t strea
   return check_launch();
 }
 
-// benchmarking switch, one value per host thread (see msgl_set_tuning)
+// benchmarking switch, one value per host thread (see msgl_set_tuning): 0 the ping-pong kernel,
+// anything else the fused kernel it replaced (8 waves x 32 rows), kept as its comparison partner
 static thread_local int t_tile_variant = 0;
 int tile_variant() { return t_tile_variant; }
 void set_tile_variant(int v) { t_tile_variant = v; }
@@ -1299,14 +1307,11 @@ int launch_prefill_tile(const PrefillArgs& a, hipStream_t stream) {
   int64_t n_blocks = 0;
   bool wide = false;
   PrefillArgs args = a;
-  if (tile_variant() != 0) args.ragged_tiles = 0;  // the fused kernels know uniform key splits only
+  if (tile_variant() != 0) args.ragged_tiles = 0;  // the fused kernel knows uniform key splits only
   const int rc = make_prefill_params(args, p, n_blocks, wide);
   if (rc != MSGL_OK || n_blocks == 0) return rc;
   const dim3 grid((unsigned)n_blocks);
-  if (tile_variant() == 1) {
-    if (wide) hipLaunchKernelGGL((prefill_tile_kernel<128, 2, 4, true>), grid, dim3(256), 0, stream, p);
-    else hipLaunchKernelGGL((prefill_tile_kernel<128, 2, 4, false>), grid, dim3(256), 0, stream, p);
-  } else if (tile_variant() == 3) {
+  if (tile_variant() != 0) {
     if (wide) hipLaunchKernelGGL((prefill_tile_kernel<128, 1, 8, true>), grid, dim3(512), 0, stream, p);
     else hipLaunchKernelGGL((prefill_tile_kernel<128, 1, 8, false>), grid, dim3(512), 0, stream, p);
   } else {
