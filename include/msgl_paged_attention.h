@@ -289,6 +289,10 @@ MSGL_API int msgl_gdn_state_inplace(const void* q, const void* k, const void* v,
  *                            and launches with one query block per request and kv head give each
  *                            request as many shares as its length asks for, up to 128 requests
  *                            or 1024 long ones)
+ *   MSGL_TUNE_PREFILL_GANGS  negative: extends with several query blocks per request and kv head
+ *                            never use gang ranges (one workgroup per compute unit for the whole
+ *                            launch, the units' keys shared out by length); 0: chosen from the sizes;
+ *                            positive: whenever the shape allows it, however small the launch
  */
 #define MSGL_TUNE_SEGMENTS 0
 #define MSGL_TUNE_MIN_SEGMENT 1
@@ -298,6 +302,7 @@ MSGL_API int msgl_gdn_state_inplace(const void* q, const void* k, const void* v,
 #define MSGL_TUNE_GDN_ROWS 5
 #define MSGL_TUNE_PREFILL_KEY_SPLITS 6
 #define MSGL_TUNE_SPLITKV_BOUNDARY 7
+#define MSGL_TUNE_PREFILL_GANGS 8
 MSGL_API int msgl_set_tuning(int32_t knob, int64_t value);
 
 #ifdef __cplusplus

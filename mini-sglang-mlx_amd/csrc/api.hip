@@ -3,6 +3,7 @@
 // paged_prefill_attention.cpp:31-76, store_kv_cache.cpp:22-63) as far as raw pointers
 // and sizes can express them; rank and dtype-equality checks live in the Python shim.
 #include <algorithm>
+#include <atomic>
 
 #include "msgl_internal.h"
 #include "prefill_params.h"
@@ -14,6 +15,9 @@ namespace {
 // always agree on the split, whatever other threads (one per stream) do.
 thread_local int64_t t_tune[3] = {0, 0, 0};
 thread_local int64_t t_key_splits = 0;
+thread_local int64_t t_gangs = 0;  // negative: never use gang ranges
+// launch numbers for the count words of gang ranges (see prefill_gangs()); never 0
+std::atomic<unsigned long long> g_gang_nonce{1};
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
@@ -106,6 +110,10 @@ int msgl_set_tuning(int32_t knob, int64_t value) {
   }
   if (knob == MSGL_TUNE_PREFILL_KEY_SPLITS) {
     t_key_splits = value < 0 ? 0 : value;
+    return MSGL_OK;
+  }
+  if (knob == MSGL_TUNE_PREFILL_GANGS) {
+    t_gangs = value;
     return MSGL_OK;
   }
   if (knob < 0 || knob > 2) return MSGL_ERR_SHAPE;
@@ -233,6 +241,14 @@ static int ragged_tiles(int64_t batch, int64_t total_kv, int64_t n_kv, int64_t g
                                     msgl::prefill_block_rows(head_dim), t_key_splits);
 }
 
+// Gang ranges for the head_dim 128 ping-pong kernel (several query blocks per (request, kv head)).
+static int gangs_for(int64_t batch, int64_t total_kv, int64_t n_kv, int64_t group, int64_t max_len_extend,
+                     int64_t head_dim, int64_t window, int key_splits) {
+  if (head_dim != 128 || msgl::tile_variant() != 0 || t_gangs < 0) return 0;
+  return msgl::prefill_gangs(batch, total_kv, n_kv, group, max_len_extend, window, msgl::kPrefillBlockRows,
+                             t_gangs > 0 ? 1 : key_splits, t_key_splits, /*whatever_the_size=*/t_gangs > 0);
+}
+
 static bool use_splitkv_route(int64_t group, int64_t max_len_extend, int64_t head_dim, int64_t batch,
                               int64_t total_kv, int64_t n_kv) {
   const int64_t cols = group * max_len_extend;
@@ -271,7 +287,11 @@ size_t msgl_paged_prefill_workspace_bytes(int64_t batch, int64_t total_q, int64_
                                                   max_len_extend, head_dim, ragged);
     const int k = msgl::prefill_key_splits(batch, total_kv, num_kv_heads, group, max_len_extend, 0,
                                            msgl::prefill_block_rows(head_dim), t_key_splits);
-    return msgl::prefill_split_workspace_bytes(total_q, num_q_heads, head_dim, k);
+    const int gangs = gangs_for(batch, total_kv, num_kv_heads, group, max_len_extend, head_dim, 0, k);
+    const size_t split_need = msgl::prefill_split_workspace_bytes(total_q, num_q_heads, head_dim, k);
+    if (gangs > 0)
+      return std::max(split_need, msgl::prefill_gang_workspace_bytes(batch, num_kv_heads, group, max_len_extend, gangs));
+    return split_need;
   }
   const size_t split_need = msgl::splitkv_workspace_bytes(
       batch, num_q_heads, num_kv_heads, head_dim, max_len_extend,
@@ -383,6 +403,20 @@ int msgl_paged_prefill_attention(const void* q, const void* k_cache, const void*
     const size_t need = msgl::prefill_split_workspace_bytes(total_q, num_q_heads, head_dim, a.key_splits);
     if (!workspace || workspace_bytes < need || !aligned16(workspace)) a.key_splits = 1;
     else a.workspace = workspace;
+  }
+  a.gangs = 0;
+  if (t_gangs > 0 && a.ragged_tiles == 0) a.key_splits = 1;  // forced for a test: gang ranges instead
+  if (a.ragged_tiles == 0 && a.key_splits == 1) {
+    const int gangs = gangs_for(batch, total_kv, num_kv_heads, group, max_len_extend, head_dim,
+                                sliding_window_size, a.key_splits);
+    // so are gang ranges: without room for their slots every unit goes to one workgroup per query block
+    if (gangs > 0 && workspace && aligned16(workspace) &&
+        workspace_bytes >= msgl::prefill_gang_workspace_bytes(batch, num_kv_heads, group, max_len_extend, gangs)) {
+      a.gangs = gangs;
+      a.workspace = workspace;
+      a.gang_nonce = g_gang_nonce.fetch_add(1, std::memory_order_relaxed) & ((1ull << 47) - 1);
+      if (a.gang_nonce == 0) a.gang_nonce = g_gang_nonce.fetch_add(1, std::memory_order_relaxed);
+    }
   }
   return head_dim == 256 ? msgl::launch_prefill_tile256(a, s) : msgl::launch_prefill_tile(a, s);
 }

@@ -79,13 +79,17 @@ struct PrefillArgs {
   // ragged shares instead (one query block per (request, kv head) only): key tiles per share,
   // 0 = off; `workspace` then holds prefill_ragged_workspace_bytes()
   int32_t ragged_tiles;
+  // gang ranges instead (several query blocks per (request, kv head), head_dim 128 only): gangs
+  // per XCD, 0 = off; `workspace` then holds prefill_gang_workspace_bytes(); `gang_nonce` is a
+  // number no earlier launch on this workspace has used
+  int32_t gangs;
+  unsigned long long gang_nonce;
 };
 int launch_prefill_tile(const PrefillArgs& a, hipStream_t stream);     // head_dim 128
 // ---- paged_prefill_d256.hip ----------------------------------------------------------
 int launch_prefill_tile256(const PrefillArgs& a, hipStream_t stream);  // head_dim 256
-// benchmarking switch: head_dim 128 kernel (0: ping-pong kernel, 3: fused kernel with 8 waves x
-// 32 rows, 1: fused kernel with 4 waves x 64 rows; all cover 256 rows per workgroup); 2 sends
-// head_dim 256 through the split-K kernel in chunks of queries instead of its tile kernel
+// benchmarking switch: head_dim 128 kernel (0: ping-pong kernel, anything else: the fused kernel
+// it replaced, 8 waves x 32 rows)
 int tile_variant();
 void set_tile_variant(int v);
 

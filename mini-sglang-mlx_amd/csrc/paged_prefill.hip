@@ -686,12 +686,43 @@ __global__ __launch_bounds__(512) void prefill_pingpong_kernel(PrefillParams p) 
   const int h = lane >> 5;
   const int c32 = lane & 31;
 
+  // ---- gang ranges: the workgroup stays for the launch and takes the parts of the units that
+  // fall into its gang's range, one after the other (see gang_plan) -----------------------------
+  __shared__ GangLds gang_lds;
+  __shared__ int gang_last;
+  const bool ganged = p.gangs > 0;
+  const int gang_xcd = (int)(blockIdx.x & 7);
+  const int gang_id = ganged ? (int)(blockIdx.x >> 3) / p.n_qblk : 0;
+  const int gang_member = ganged ? (int)(blockIdx.x >> 3) % p.n_qblk : 0;
+  GangPlan plan{0, 0, 0, 0};
+  if (ganged) plan = gang_plan<NW * 64>(p, gang_lds, gang_xcd, gang_id, gang_member, kRows, tid);
+  for (int piece = plan.first_unit;; ++piece) {
   // ---- block -> (request, kv head, key split, q block): as in prefill_tile_kernel; with ragged
-  // shares, block -> (unit = (request, share), kv head) ----------------------------------------
-  int b, kvh, split, qblk, n_shares = 1;
+  // shares, block -> (unit = (request, share), kv head); with gang ranges, the next unit of the
+  // range -------------------------------------------------------------------------------------
+  int b, kvh, split = 0, qblk, n_shares = 1;
   bool to_partial = p.n_ksplit > 1;  // leave a partial for the merge kernel, not the result
   int64_t part_at = 0;               // partial row of the block's row 0 (ragged shares)
-  if (p.ragged_tiles > 0) {
+  int piece_a = 0, piece_b = 0x7fffff, unit_start = 0, unit_tiles = 0;  // gang ranges: tiles [a, b) of the unit
+  bool piece_whole = true;
+  if (ganged) {
+    if (piece > plan.last_unit) break;
+    // the stages double as the staging area of the previous part's output: read out by now
+    if (piece > plan.first_unit) __syncthreads();
+    unit_tiles = __builtin_amdgcn_readfirstlane(gang_lds.len[piece]);
+    unit_start = __builtin_amdgcn_readfirstlane(gang_lds.start[piece]);
+    piece_a = max(plan.lo - unit_start, 0);
+    piece_b = min(plan.hi - unit_start, unit_tiles);
+    if (piece_b <= piece_a) continue;
+    piece_whole = piece_a == 0 && piece_b == unit_tiles;
+    const int unit = piece * 8 + gang_xcd;
+    b = __builtin_amdgcn_readfirstlane(gang_lds.order[unit / p.n_kv]);
+    kvh = unit % p.n_kv;
+    qblk = gang_member;
+    to_partial = false;
+  } else if (piece > 0) {
+    break;
+  } else if (p.ragged_tiles > 0) {
     kvh = (int)(blockIdx.x % (unsigned)p.n_kv);
     const int u = (int)(blockIdx.x / (unsigned)p.n_kv);
     const RaggedUnit ru = ragged_unit<NW * 64>(p, u, tid);
@@ -717,14 +748,19 @@ __global__ __launch_bounds__(512) void prefill_pingpong_kernel(PrefillParams p) 
     b = request_of_rank<NW * 64>(p.kv_indptr, p.batch, want_rank, tid);
   }
 
-  const int q_start = p.qo_indptr[b];
-  const int q_len = min(p.qo_indptr[b + 1] - q_start, p.max_len_extend);
-  const int kv_start = p.kv_indptr[b];
-  const int kn = max(p.kv_indptr[b + 1] - kv_start, 0);
-  const int prefix = p.prefix_lens[b];
+  // (gang ranges keep every request's geometry in LDS: a part starts without a memory round trip)
+  auto uniform = [](int x) { return __builtin_amdgcn_readfirstlane(x); };  // the same in every lane: a scalar
+  const int q_start = ganged ? uniform(gang_lds.q_start[b]) : p.qo_indptr[b];
+  const int q_len = ganged ? uniform(gang_lds.q_len[b]) : min(p.qo_indptr[b + 1] - q_start, p.max_len_extend);
+  const int kv_start = ganged ? uniform(gang_lds.kv_start[b]) : p.kv_indptr[b];
+  const int kn = ganged ? uniform(gang_lds.kv_len[b]) : max(p.kv_indptr[b + 1] - kv_start, 0);
+  const int prefix = ganged ? uniform(gang_lds.prefix[b]) : p.prefix_lens[b];
   const int rows_total = q_len * p.group;
   const int row0 = qblk * kRows;
-  if (row0 >= rows_total) return;
+  if (row0 >= rows_total) {
+    if (ganged) continue;  // this request has no such query block
+    return;
+  }
 
   const bool idle = __builtin_amdgcn_readfirstlane(row0 + w * 32 >= rows_total ? 1 : 0) != 0;
   const int qi_lo = row0 / p.group;
@@ -733,7 +769,11 @@ __global__ __launch_bounds__(512) void prefill_pingpong_kernel(PrefillParams p) 
   int k_lo = (p.window > 0) ? max(0, prefix + qi_lo - p.window + 1) : 0;
   k_lo &= ~(kBN - 1);
   if (k_hi < k_lo) k_hi = k_lo;
-  if (p.ragged_tiles > 0) {  // the request's shares are equal: none longer than ragged_tiles
+  if (ganged) {  // tiles [piece_a, piece_b) of the unit, as far as this query block sees them
+    k_lo = min(k_lo + piece_a * kBN, k_hi);
+    k_hi = min(k_hi, piece_b * kBN);
+    if (k_hi < k_lo) k_hi = k_lo;
+  } else if (p.ragged_tiles > 0) {  // the request's shares are equal: none longer than ragged_tiles
     const int all_tiles = (k_hi - k_lo + kBN - 1) / kBN;
     const int share = (all_tiles + n_shares - 1) / n_shares * kBN;
     k_lo = min(k_lo + split * share, k_hi);
@@ -1126,6 +1166,86 @@ __global__ __launch_bounds__(512) void prefill_pingpong_kernel(PrefillParams p) 
     // epilogue reuses the stages as its output staging area
   }
 
+  // ---- gang ranges: a part of a unit.  Its unnormalised rows, row references and row sums go to
+  // the part's slot (lane-major: the only reader has this kernel's register layout), the workgroup
+  // counts itself, and the part that counts last adds the others to its registers and goes on to
+  // write the result.  Slots and counts are read and written at agent scope (parts of a unit
+  // may sit on different XCDs as far as the program is concerned; nothing here relies on the
+  // order in which the parts finish, and nobody waits for anybody).
+  if (ganged && !piece_whole) {
+    auto slot_of = [&](int g) {
+      const int64_t at = (((int64_t)gang_xcd * p.gangs + g) * 2 + gang_slot_of(gang_lds, g, unit_start)) * p.n_qblk + gang_member;
+      return reinterpret_cast<unsigned long long*>(p.gang_slots) + at * (int64_t)(kGangSlotBytes / 8);
+    };
+    auto pair_bits = [](float x, float y) {
+      return (unsigned long long)__builtin_bit_cast(uint32_t, x) | ((unsigned long long)__builtin_bit_cast(uint32_t, y) << 32);
+    };
+    {
+      unsigned long long* mine = slot_of(gang_id);
+      unsigned long long* o64 = mine + (int64_t)w * 32 * kWave + lane;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int i = 0; i < 16; i += 2)
+          __hip_atomic_store(o64 + (dt * 8 + i / 2) * kWave, pair_bits(oacc[dt][i], oacc[dt][i + 1]), __ATOMIC_RELAXED,
+                             __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(mine + 8 * 32 * kWave + w * kWave + lane, pair_bits(m_run, l_run), __ATOMIC_RELAXED,
+                         __HIP_MEMORY_SCOPE_AGENT);
+    }
+    // count word = launch number << 16 | parts done; a word from another launch counts as zero.
+    // It is read while the slot's stores drain (the update below then usually succeeds at once).
+    unsigned long long* cnt = p.gang_counts + ((int64_t)(piece * 8 + gang_xcd) * p.n_qblk + gang_member);
+    unsigned long long seen = 0;
+    if (tid == 0) seen = __hip_atomic_load(cnt, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    wait_all_vm();  // the slot is written before the workgroup counts itself
+    __syncthreads();
+    if (tid == 0) {
+      int n_parts = 0;
+      for (int g = 0; g < p.gangs; ++g)
+        n_parts += (gang_lds.cuts[g] < unit_start + unit_tiles && gang_lds.cuts[g + 1] > unit_start &&
+                    gang_lds.cuts[g + 1] > gang_lds.cuts[g]) ? 1 : 0;
+      unsigned long long want;
+      do {
+        want = ((seen >> 16) == p.gang_nonce ? seen : (p.gang_nonce << 16)) + 1;
+      } while (!__hip_atomic_compare_exchange_strong(cnt, &seen, want, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
+                                                     __HIP_MEMORY_SCOPE_AGENT));
+      const bool last = (int)(want & 0xffff) == n_parts;
+      // the last part leaves the word as a launch that never happened (a replayed launch
+      // carries the same number)
+      if (last) __hip_atomic_store(cnt, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      gang_last = last ? 1 : 0;
+    }
+    __syncthreads();
+    if (gang_last == 0) continue;
+    for (int g = 0; g < p.gangs; ++g) {
+      if (g == gang_id || !(gang_lds.cuts[g] < unit_start + unit_tiles && gang_lds.cuts[g + 1] > unit_start &&
+                            gang_lds.cuts[g + 1] > gang_lds.cuts[g]))
+        continue;
+      const unsigned long long* theirs = slot_of(g);
+      const unsigned long long* o64 = theirs + (int64_t)w * 32 * kWave + lane;
+      unsigned long long got[32];
+#pragma unroll
+      for (int j = 0; j < 32; ++j) got[j] = __hip_atomic_load(o64 + j * kWave, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const unsigned long long ml = __hip_atomic_load(theirs + 8 * 32 * kWave + w * kWave + lane, __ATOMIC_RELAXED,
+                                                      __HIP_MEMORY_SCOPE_AGENT);
+      const float m_other = __builtin_bit_cast(float, (uint32_t)ml);
+      const float l_other = __builtin_bit_cast(float, (uint32_t)(ml >> 32));
+      const float m_new = fmaxf(m_run, m_other);
+      const float m_ref = (m_new == kNegInf) ? 0.f : m_new;
+      const float a_mine = fast_exp2(m_run - m_ref), a_other = fast_exp2(m_other - m_ref);
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int i = 0; i < 16; i += 2) {
+          const unsigned long long v = got[dt * 8 + i / 2];
+          oacc[dt][i] = oacc[dt][i] * a_mine + a_other * __builtin_bit_cast(float, (uint32_t)v);
+          oacc[dt][i + 1] = oacc[dt][i + 1] * a_mine + a_other * __builtin_bit_cast(float, (uint32_t)(v >> 32));
+        }
+      l_run = l_run * a_mine + l_other * a_other;
+      m_run = m_new;
+    }
+  }
+
   // accumulator i of O^T tile dt is dim 32dt + 8(i/4) + 4h + i%4 of query row c32
   float l = l_run;
   l += __shfl_xor(l, 32, kWave);
@@ -1177,6 +1297,7 @@ __global__ __launch_bounds__(512) void prefill_pingpong_kernel(PrefillParams p) 
       st_global_b128(p.out + ((int64_t)(q_start + qi) * p.n_q + kvh * p.group + hh) * D + c * 8, v);
     }
   }
+  }  // the next part of the gang's range (a launch without gang ranges leaves here)
 }
 
 
@@ -1307,7 +1428,10 @@ int launch_prefill_tile(const PrefillArgs& a, hipStream_t stream) {
   int64_t n_blocks = 0;
   bool wide = false;
   PrefillArgs args = a;
-  if (tile_variant() != 0) args.ragged_tiles = 0;  // the fused kernel knows uniform key splits only
+  if (tile_variant() != 0) {  // the fused kernel knows uniform key splits only
+    args.ragged_tiles = 0;
+    args.gangs = 0;
+  }
   const int rc = make_prefill_params(args, p, n_blocks, wide);
   if (rc != MSGL_OK || n_blocks == 0) return rc;
   const dim3 grid((unsigned)n_blocks);

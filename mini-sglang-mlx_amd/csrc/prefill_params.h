@@ -31,6 +31,13 @@ struct PrefillParams {
   // (request, share), and req_units[2 b], [2 b + 1] = request b's first unit and unit count
   int32_t ragged_tiles, ragged_units, ragged_rows;
   int32_t* req_units;
+  // gang ranges (see prefill_gangs()): `gangs` per XCD, 0 = off; cuts closer than `gang_snap`
+  // tiles to either end of a (request, kv head) move to that end; a workgroup that ends up with
+  // part of a unit's keys leaves its rows in `gang_slots` and counts itself in `gang_counts`
+  int32_t gangs, gang_snap;
+  float* gang_slots;
+  unsigned long long* gang_counts;
+  unsigned long long gang_nonce;
 };
 
 constexpr int kBN = 64;  // keys per tile
@@ -148,6 +155,45 @@ inline size_t prefill_ragged_workspace_bytes(int64_t batch, int64_t total_kv, in
   return rows * (size_t)(head_dim + 1) * sizeof(float) + (size_t)batch * 2 * sizeof(int32_t);
 }
 
+// Gang ranges, for launches with several query blocks per (request, kv head) (chunked extends on
+// long prefixes: their cost is the MFMA work, and it differs from unit to unit with the prefix).
+// One workgroup per compute unit stays for the whole launch.  The 32 workgroups on an XCD form
+// 32 / n_qblk gangs; a gang's workgroups take the query blocks of one unit side by side (they read
+// the same keys at the same time: one L2 serves them) and the gangs share the XCD's units by
+// length: the units' key tiles, laid end to end, are cut into equal ranges, one per gang, so
+// every gang has the same MFMA work whatever the prefix lengths are.  A unit that a cut goes
+// through is finished by the gang that gets there last: each of its parts leaves unnormalised
+// rows, row maxima and row sums in its slot and counts itself; the part that counts last adds the
+// others to its registers and writes the result.  Returns gangs per XCD, 0 when the launch does
+// not qualify (the host knows sizes, not lengths).
+constexpr int kGangMaxUnits = 256;   // units per XCD
+constexpr int kGangMinTiles = 48;    // key tiles per gang below which one pass per unit is kept
+inline int prefill_gangs(int64_t batch, int64_t total_kv, int64_t n_kv, int64_t group,
+                         int64_t max_len_extend, int64_t window, int block_rows, int key_splits,
+                         int64_t forced_splits, bool whatever_the_size = false) {
+  if (forced_splits > 0 || key_splits > 1 || window > 0 || batch <= 0 || batch > kRankedBatch) return 0;
+  const int64_t n_qblk = (max_len_extend * group + block_rows - 1) / block_rows;
+  constexpr int64_t kUnitsPerXcd = kComputeUnits / 8;
+  if (n_qblk < 2 || n_qblk > 16 || kUnitsPerXcd % n_qblk != 0) return 0;
+  const int64_t n_pairs = batch * n_kv;
+  if (n_pairs % 8 != 0 || n_pairs / 8 > kGangMaxUnits) return 0;
+  const int64_t gangs = kUnitsPerXcd / n_qblk;
+  if (whatever_the_size) return (int)gangs;
+  if (n_pairs / 8 < gangs) return 0;  // fewer units than gangs: key splits are the tool
+  const int64_t tiles_per_xcd = prefill_tiles_bound(batch, total_kv) * n_kv / 8;
+  if (tiles_per_xcd < gangs * kGangMinTiles) return 0;
+  return (int)gangs;
+}
+constexpr size_t kGangSlotBytes = (size_t)kPrefillBlockRows * 128 * sizeof(float) + 8 * 64 * 2 * sizeof(float);
+inline size_t prefill_gang_workspace_bytes(int64_t batch, int64_t n_kv, int64_t group,
+                                           int64_t max_len_extend, int gangs) {
+  if (gangs <= 0) return 0;
+  const int64_t n_qblk = (max_len_extend * group + kPrefillBlockRows - 1) / kPrefillBlockRows;
+  const size_t slots = (size_t)8 * gangs * 2 * n_qblk;
+  const size_t counts = (size_t)batch * n_kv * n_qblk;
+  return slots * kGangSlotBytes + (counts * sizeof(unsigned long long) + 255) / 256 * 256;
+}
+
 inline size_t prefill_split_workspace_bytes(int64_t total_q, int64_t n_q, int64_t head_dim, int n_ksplit) {
   if (n_ksplit <= 1) return 0;
   return (size_t)n_ksplit * (size_t)total_q * (size_t)n_q * (size_t)(head_dim + 1) * sizeof(float);
@@ -191,6 +237,11 @@ inline int make_prefill_params(const PrefillArgs& a, PrefillParams& p, int64_t& 
   p.ragged_units = 0;
   p.ragged_rows = 0;
   p.req_units = nullptr;
+  p.gangs = 0;
+  p.gang_snap = 0;
+  p.gang_slots = nullptr;
+  p.gang_counts = nullptr;
+  p.gang_nonce = 0;
   if (a.ragged_tiles > 0 && n_qblk == 1) {
     const int64_t units = prefill_ragged_units(a.batch, a.total_kv, a.ragged_tiles);
     p.n_ksplit = 1;
@@ -224,6 +275,18 @@ inline int make_prefill_params(const PrefillArgs& a, PrefillParams& p, int64_t& 
   if (n_blocks > 0x7fffffffLL) return MSGL_ERR_SHAPE;
   p.n_qblk = (int32_t)n_qblk;
   p.n_pairs = (int32_t)n_pairs;
+  if (a.gangs > 0 && p.n_ksplit == 1 && block_rows == kPrefillBlockRows) {
+    if (!a.workspace) return MSGL_ERR_WORKSPACE;
+    p.gangs = a.gangs;
+    // the last rows' diagonal lies in the last ceil(extend / 64) tiles of a unit: no cut goes there,
+    // so every part of a unit holds keys that every row of every query block sees
+    p.gang_snap = (int32_t)((a.max_len_extend + kBN - 1) / kBN + 2);
+    const size_t slots = (size_t)8 * a.gangs * 2 * n_qblk;
+    p.gang_slots = static_cast<float*>(a.workspace);
+    p.gang_counts = reinterpret_cast<unsigned long long*>(static_cast<char*>(a.workspace) + slots * kGangSlotBytes);
+    p.gang_nonce = a.gang_nonce;
+    n_blocks = kComputeUnits;  // one workgroup per compute unit, 32 per XCD
+  }
   // narrow offsets: slot * row_bytes fits 32 bits and both factors fit 24 bits (one
   // full-rate 24-bit multiply per row)
   wide = (uint64_t)a.num_slots * (uint64_t)a.k_stride0 * 2u >= (1ull << 32) ||

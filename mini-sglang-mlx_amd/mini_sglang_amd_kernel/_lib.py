@@ -87,6 +87,7 @@ TUNE_SPLITKV_WAVES = 4
 TUNE_GDN_ROWS = 5
 TUNE_PREFILL_KEY_SPLITS = 6
 TUNE_SPLITKV_BOUNDARY = 7
+TUNE_PREFILL_GANGS = 8
 
 _lib = None
 

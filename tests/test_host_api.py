@@ -73,9 +73,17 @@ def test_c_abi_argument_checks_return_codes_without_touching_a_gpu():
     assert lib.msgl_set_tuning(99, 1) == -9
     assert lib.msgl_paged_decode_workspace_bytes(4, 1000, 32, 8, 128) > 0
     assert lib.msgl_paged_decode_workspace_bytes(4, 1000, 30, 8, 128) == 0
-    # prefill workspace: none for a launch that fills the chip, the partials of a key split for
-    # one long request, none again when splitting is switched off
+    # prefill workspace: the slots and count words of gang ranges for a launch with several query
+    # blocks per (request, kv head) that fills the chip (8 XCDs x 4 gangs x 2 slots x 8 query blocks
+    # of 256 rows x 128 floats + 8 waves x 64 lanes x 2 floats; one 8-byte count per (request, kv
+    # head, query block)), nothing when they are switched off or at head_dim 256; the partials of a
+    # key split for one long request, none again when splitting is switched off
+    slot = 256 * 128 * 4 + 8 * 64 * 2 * 4
+    assert lib.msgl_paged_prefill_workspace_bytes(8, 4096, 8 * 8704, 32, 8, 128, 512) == 8 * 4 * 2 * 8 * slot + 8 * 8 * 8 * 8
+    assert lib.msgl_set_tuning(8, -1) == 0
     assert lib.msgl_paged_prefill_workspace_bytes(8, 4096, 8 * 8704, 32, 8, 128, 512) == 0
+    assert lib.msgl_set_tuning(8, 0) == 0
+    assert lib.msgl_paged_prefill_workspace_bytes(8, 4096, 8 * 8704, 32, 8, 256, 512) == 0
     one_long = (1, 512, 32768 + 512, 32, 8, 128, 512)
     need = lib.msgl_paged_prefill_workspace_bytes(*one_long)
     assert need > 0 and need % (512 * 32 * (128 + 1) * 4) == 0
