@@ -154,8 +154,10 @@ def test_uniform_attention_closed_form_every_row_full_size(gpu, cfg, variant):
     """Full size, every request, every row and head, against a closed form: q = 0 makes the
     weights exactly 1 / (visible keys), so a dropped, doubled or wrongly gathered key, a
     wrong causal limit or window floor, or a mis-merged segment moves the result by about
-    |v| / keys, which the bound below (bf16 rounding of the result plus 2e-5) does not cover
-    for a v of ordinary size."""
+    |v| / keys, which the bound below (bf16 rounding of the result plus 4e-5) does not cover
+    for a v of ordinary size.  (4e-5: where the partials of a request's shares are much larger
+    than their mean, which is what q = 0 on random V produces, their rounding to IEEE half,
+    2^-12 of a partial of 0.05 .. 0.1, is what is left of the error.)"""
     print(f"cfg{cfg} {variant} uniform attention: build", flush=True)
     wl = _full_size_workload(cfg, variant, gpu)
     wl.q.zero_()
@@ -163,7 +165,7 @@ def test_uniform_attention_closed_form_every_row_full_size(gpu, cfg, variant):
     print(f"cfg{cfg} {variant} uniform attention: closed form", flush=True)
     want = _uniform_attention_expected(g)
     diff = (got.to(gpu).double() - want).abs()
-    bound = want.abs() * 2.0 ** -8 + 2e-5
+    bound = want.abs() * 2.0 ** -8 + 4e-5
     worst = float((diff - bound).max())
     assert worst <= 0.0, (f"cfg{cfg} {variant}: a row is {worst:.3e} beyond its bound; "
                           f"max-abs diff {float(diff.max()):.3e}")
@@ -257,7 +259,7 @@ def test_few_long_requests_merge_of_many_partials(gpu, lens, ext, head_dim):
     got, _ = run_gpu(g, gpu, store=False)
     want = _uniform_attention_expected(g)
     diff = (got.to(gpu).double().reshape(want.shape) - want).abs()
-    assert float((diff - (want.abs() * 2.0 ** -8 + 2e-5)).max()) <= 0.0, (
+    assert float((diff - (want.abs() * 2.0 ** -8 + 4e-5)).max()) <= 0.0, (
         f"uniform attention: max-abs diff {float(diff.max()):.3e}")
     q, want = _needle_queries(g)
     g.q = q.reshape(q_rand.shape)
