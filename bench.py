@@ -50,16 +50,23 @@ def time_steps(fn, steps: int, warmup: int, spinup_ms: float = SPINUP_MS):
     whether the first one still saw the clocks settling."""
     import torch
 
+    probe = _ClockProbe()
+
     def loop_ms():
         e0 = torch.cuda.Event(enable_timing=True)
         e1 = torch.cuda.Event(enable_timing=True)
+        probe.arm()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         e0.record()
-        for _ in range(steps):
-            fn()
+        try:
+            for _ in range(steps):
+                fn()
+        finally:
+            probe.disarm()
         e1.record()
         torch.cuda.synchronize()
+        time_steps.last_shader_ghz = probe.ghz()
         return e0.elapsed_time(e1), (time.perf_counter() - t0) * 1e3
 
     # The shader clock needs some tens of milliseconds of load to settle (measured: the MFMA
@@ -86,9 +93,37 @@ def time_steps(fn, steps: int, warmup: int, spinup_ms: float = SPINUP_MS):
         ends[i].record()
     torch.cuda.synchronize()
     per = [s.elapsed_time(e) for s, e in zip(starts, ends)]
+    ghz = time_steps.last_shader_ghz  # of the reported pass
     again, _ = loop_ms()
     time_steps.last_repeat_ms = again / steps
+    time_steps.last_shader_ghz = ghz
     return loop / steps, per, wall_ms
+
+
+class _ClockProbe:
+    """Shader clock under the attention kernels of a timed loop: the library's measurement aid
+    (MSGL_TUNE_CLOCK_PROBE) makes workgroup 0 of every attention kernel leave the shader cycles
+    and the 100 MHz wall ticks it lived for in two device words; read after the loop, they are
+    those of its last launch."""
+
+    def __init__(self):
+        import torch
+
+        from mini_sglang_amd_kernel import _lib
+
+        self._lib = _lib
+        self.buf = torch.zeros(2, dtype=torch.int64, device="cuda")
+
+    def arm(self):
+        self.buf.zero_()
+        self._lib.set_tuning(self._lib.TUNE_CLOCK_PROBE, self.buf.data_ptr())
+
+    def disarm(self):
+        self._lib.set_tuning(self._lib.TUNE_CLOCK_PROBE, 0)
+
+    def ghz(self):
+        cycles, ticks = self.buf.tolist()
+        return cycles / ticks * 0.1 if ticks > 0 else None
 
 
 def make_step(g):
@@ -177,6 +212,8 @@ def run_config(cfg: int, variant: str, steps: int, warmup: int, check: bool, cpu
         "sliding_window": wl.sliding_window_size,
         "ms_mean": mean_ms, "ms_median": med_ms, "ms_min": min(per),
         "ms_mean_repeat": time_steps.last_repeat_ms, "spinup_ms": SPINUP_MS,
+        # shader clock under the attention kernel of the last timed step (None: no such kernel ran)
+        "shader_ghz": time_steps.last_shader_ghz,
         "per_step_us": [round(x * 1e3, 1) for x in per],
         "wall_ms_per_step": wall_ms / steps, "steps": steps, "warmup": warmup,
         "algorithmic_bytes": abytes, "algorithmic_flops": aflops, "store_bytes": sbytes,
@@ -589,10 +626,12 @@ def run_small_launch_extends(dev, steps: int, warmup: int):
         outs = {}
         for label, knob in (("one_pass", 1), ("key_split", 0)):
             _lib.set_tuning(_lib.TUNE_PREFILL_KEY_SPLITS, knob)
-            ms, _, _ = time_steps(step, max(3, steps // 5), max(1, warmup // 5))
-            outs[label] = step().float()
-            torch.cuda.synchronize()
-            _lib.set_tuning(_lib.TUNE_PREFILL_KEY_SPLITS, 0)
+            try:  # whatever happens, the later legs run with the library's own choice
+                ms, _, _ = time_steps(step, max(3, steps // 5), max(1, warmup // 5))
+                outs[label] = step().float()
+                torch.cuda.synchronize()
+            finally:
+                _lib.set_tuning(_lib.TUNE_PREFILL_KEY_SPLITS, 0)
             row[label + "_us"] = ms * 1e3
             row[label + "_TFLOPs"] = row["algorithmic_flops"] / (ms * 1e-3) / 1e12
         row["max_abs_diff"] = float((outs["one_pass"] - outs["key_split"]).abs().max())
@@ -788,9 +827,10 @@ def main():
         rows.append(row)
         perf = (f"{row['achieved_TBps']:.3f} TB/s" if row["bound"] == "hbm"
                 else f"{row['achieved_TFLOPs']:.1f} TFLOP/s")
+        clock = f"  shader clock {row['shader_ghz']:.2f} GHz" if row.get("shader_ghz") else ""
         log(f"[cfg {tok}] {row['workload']}: {row['ms_mean']*1e3:.1f} us mean "
             f"({row['ms_min']*1e3:.1f} min)  {perf}  {row['roofline_frac']*100:.1f}% of "
-            f"{row['bound']} peak  err max {row.get('max_abs_err', float('nan')):.2e} "
+            f"{row['bound']} peak{clock}  err max {row.get('max_abs_err', float('nan')):.2e} "
             f"mean {row.get('mean_abs_err', float('nan')):.2e}  cpu "
             f"{row.get('cpu_baseline', {}).get('value', float('nan')):.4f} "
             f"{row.get('cpu_baseline', {}).get('unit', '')}")

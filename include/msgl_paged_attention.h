@@ -293,6 +293,10 @@ MSGL_API int msgl_gdn_state_inplace(const void* q, const void* k, const void* v,
  *                            never use gang ranges (one workgroup per compute unit for the whole
  *                            launch, the units' keys shared out by length); 0: chosen from the sizes;
  *                            positive: whenever the shape allows it, however small the launch
+ *   MSGL_TUNE_CLOCK_PROBE    measurement aid: the value is a device pointer to two int64 (0: none).
+ *                            Workgroup 0 of every attention kernel launched by this thread then
+ *                            leaves there the shader cycles and the 100 MHz wall ticks it lived
+ *                            for: cycles / ticks x 0.1 = the shader clock in GHz under that kernel
  */
 #define MSGL_TUNE_SEGMENTS 0
 #define MSGL_TUNE_MIN_SEGMENT 1
@@ -303,6 +307,7 @@ MSGL_API int msgl_gdn_state_inplace(const void* q, const void* k, const void* v,
 #define MSGL_TUNE_PREFILL_KEY_SPLITS 6
 #define MSGL_TUNE_SPLITKV_BOUNDARY 7
 #define MSGL_TUNE_PREFILL_GANGS 8
+#define MSGL_TUNE_CLOCK_PROBE 9
 MSGL_API int msgl_set_tuning(int32_t knob, int64_t value);
 
 #ifdef __cplusplus

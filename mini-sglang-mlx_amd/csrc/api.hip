@@ -16,6 +16,7 @@ namespace {
 thread_local int64_t t_tune[3] = {0, 0, 0};
 thread_local int64_t t_key_splits = 0;
 thread_local int64_t t_gangs = 0;  // negative: never use gang ranges
+thread_local long long* t_clock_probe = nullptr;
 // launch numbers for the count words of gang ranges (see prefill_gangs()); never 0
 std::atomic<unsigned long long> g_gang_nonce{1};
 
@@ -63,6 +64,10 @@ int32_t segments(int64_t total_kv, int64_t n_kv, int64_t head_dim, int64_t cols)
 int64_t smallq_base_cols(int64_t head_dim) { return head_dim == 128 ? 48 : 16; }
 
 }  // namespace
+
+namespace msgl {
+long long* clock_probe() { return t_clock_probe; }
+}  // namespace msgl
 
 extern "C" {
 
@@ -114,6 +119,10 @@ int msgl_set_tuning(int32_t knob, int64_t value) {
   }
   if (knob == MSGL_TUNE_PREFILL_GANGS) {
     t_gangs = value;
+    return MSGL_OK;
+  }
+  if (knob == MSGL_TUNE_CLOCK_PROBE) {
+    t_clock_probe = reinterpret_cast<long long*>(static_cast<intptr_t>(value));
     return MSGL_OK;
   }
   if (knob < 0 || knob > 2) return MSGL_ERR_SHAPE;

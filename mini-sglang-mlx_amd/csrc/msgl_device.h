@@ -98,6 +98,28 @@ __device__ __forceinline__ float wave_max_xor(float v, int mask) {
 
 __device__ __forceinline__ int lane_id() { return threadIdx.x & (kWave - 1); }
 
+// Measurement aid: when `dst` is given, thread 0 of workgroup 0 leaves the shader cycles and the
+// 100 MHz wall ticks between its construction and its destruction (every way out of the kernel) in
+// dst[0], dst[1]: cycles / ticks x 0.1 is the shader clock in GHz while the kernel ran.  (Both
+// counters are read by the same wave: the cycle counters of different compute units are unrelated.)
+struct ClockProbe {
+  long long* dst;
+  long long c0, w0;
+  __device__ __forceinline__ explicit ClockProbe(long long* d)
+      : dst((d != nullptr && blockIdx.x == 0 && threadIdx.x == 0) ? d : nullptr), c0(0), w0(0) {
+    if (dst != nullptr) {
+      c0 = clock64();
+      w0 = wall_clock64();
+    }
+  }
+  __device__ __forceinline__ ~ClockProbe() {
+    if (dst != nullptr) {
+      dst[0] = clock64() - c0;
+      dst[1] = wall_clock64() - w0;
+    }
+  }
+};
+
 // Inclusive prefix sum over the 64 lanes of a wave.
 __device__ __forceinline__ int wave_inclusive_scan(int v) {
   const int lane = lane_id();

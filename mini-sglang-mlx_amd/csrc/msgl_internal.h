@@ -92,6 +92,9 @@ int launch_prefill_tile256(const PrefillArgs& a, hipStream_t stream);  // head_d
 // it replaced, 8 waves x 32 rows)
 int tile_variant();
 void set_tile_variant(int v);
+// measurement aid (MSGL_TUNE_CLOCK_PROBE): two device int64 the attention kernels' workgroup 0
+// fills with its shader cycles and 100 MHz wall ticks, or nullptr; one value per host thread
+long long* clock_probe();
 
 // ---- build_metadata.hip ------------------------------------------------------------
 struct MetadataArgs {

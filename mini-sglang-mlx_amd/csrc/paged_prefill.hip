@@ -679,6 +679,7 @@ __global__ __launch_bounds__(512) void prefill_pingpong_kernel(PrefillParams p) 
   static_assert(kRows * OROW * 2 <= pp::kSmem, "output staging must fit the stages");
   __shared__ __attribute__((aligned(16))) unsigned char smem[pp::kSmem];
   using OffT = typename std::conditional<WIDE, uint64_t, uint32_t>::type;
+  const ClockProbe clock_probe_(p.clock_probe);
 
   const int tid = threadIdx.x;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);

@@ -60,6 +60,7 @@ __global__ __launch_bounds__(kNW * 64) void prefill_tile256_kernel(PrefillParams
   constexpr int SMEM_BYTES = kStageTotal > O_BYTES ? kStageTotal : O_BYTES;
   __shared__ __attribute__((aligned(16))) unsigned char smem[SMEM_BYTES];
   using OffT = typename std::conditional<WIDE, uint64_t, uint32_t>::type;
+  const ClockProbe clock_probe_(p.clock_probe);
 
   const int tid = threadIdx.x;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);

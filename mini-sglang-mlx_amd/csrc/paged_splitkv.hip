@@ -71,6 +71,7 @@ struct SplitKvParams {
   int32_t wide;  // pool byte offsets need 64 bits
   uint32_t max_slot;  // num_slots - 1: slot ids are clamped to it before they become addresses
   float scale_log2e;
+  long long* clock_probe;  // measurement aid, see ClockProbe; nullptr: off
 };
 
 // Visible key range and query geometry of one request.
@@ -220,6 +221,7 @@ template <int D, int NCT, int NW, bool WIDE, bool F16>
 __global__ __launch_bounds__(64 * NW, ((D == 128 && NCT == 1) ? 2 : 1)) void splitkv_attention_kernel(SplitKvParams p) {
   constexpr int KS = D / 32;   // k-steps of the QK product
   constexpr int VH = D / 128;  // 128-wide halves of D in the PV product
+  const ClockProbe clock_probe_(p.clock_probe);
   const int lane = lane_id();
   const int t16 = lane & 15;
   const int g = lane >> 4;
@@ -920,6 +922,7 @@ int launch_splitkv(const SplitKvArgs& a, hipStream_t stream) {
   p.is_cross = a.is_cross;
   p.window = a.window;
   p.scale_log2e = a.sm_scale * kLog2e;
+  p.clock_probe = clock_probe();
   p.wide = ((uint64_t)a.num_slots * (uint64_t)a.k_stride0 * 2u >= (1ull << 32) ||
             (uint64_t)a.num_slots * (uint64_t)a.v_stride0 * 2u >= (1ull << 32)) ? 1 : 0;
   if ((int64_t)p.n_seg * p.head_groups > 0x7fffffffLL) return MSGL_ERR_SHAPE;

@@ -38,6 +38,7 @@ struct PrefillParams {
   float* gang_slots;
   unsigned long long* gang_counts;
   unsigned long long gang_nonce;
+  long long* clock_probe;  // measurement aid, see ClockProbe; nullptr: off
 };
 
 constexpr int kBN = 64;  // keys per tile
@@ -242,6 +243,7 @@ inline int make_prefill_params(const PrefillArgs& a, PrefillParams& p, int64_t& 
   p.gang_slots = nullptr;
   p.gang_counts = nullptr;
   p.gang_nonce = 0;
+  p.clock_probe = clock_probe();
   if (a.ragged_tiles > 0 && n_qblk == 1) {
     const int64_t units = prefill_ragged_units(a.batch, a.total_kv, a.ragged_tiles);
     p.n_ksplit = 1;

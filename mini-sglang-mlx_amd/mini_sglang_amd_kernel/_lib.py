@@ -88,6 +88,7 @@ TUNE_GDN_ROWS = 5
 TUNE_PREFILL_KEY_SPLITS = 6
 TUNE_SPLITKV_BOUNDARY = 7
 TUNE_PREFILL_GANGS = 8
+TUNE_CLOCK_PROBE = 9
 
 _lib = None
 

@@ -22,7 +22,7 @@ def gpu():
     return torch.device("cuda:0")
 
 
-_KNOBS = range(9)  # MSGL_TUNE_* of include/msgl_paged_attention.h
+_KNOBS = range(10)  # MSGL_TUNE_* of include/msgl_paged_attention.h
 
 
 def _reset_knobs():
