@@ -150,9 +150,15 @@ MSGL_API int msgl_paged_decode_attention_noalloc(const void* q, const void* k_ca
 /*
  * Workspace (bytes) that msgl_paged_prefill_attention needs for these sizes: the partials of the
  * split-K route, or those of the tile kernels when the launch is too small to fill the chip and
- * the keys of each query block are shared out over several workgroups; 0 otherwise.  The split-K
+ * the keys of each query block are shared out over several workgroups, or (head_dim 128, 2, 4, 8
+ * or 16 query blocks of 256 rows per request and kv head, enough work to fill the chip) the
+ * slots and count words of gang ranges, with which one workgroup per compute unit stays for the
+ * launch and the (request, kv head) units are shared out by length; 0 otherwise.  The split-K
  * route needs its workspace (MSGL_ERR_WORKSPACE without it); the tile kernels fall back to one
- * pass over the keys when the workspace is missing or too small.
+ * pass over the keys per query block when the workspace is missing or too small.  total_kv must
+ * be at least kv_indptr[batch], here and in msgl_paged_prefill_attention: key shares, grids and
+ * this size are derived from it (a smaller value leaves requests' rows unwritten).  Nothing in
+ * the workspace has to be initialised.
  */
 MSGL_API size_t msgl_paged_prefill_workspace_bytes(int64_t batch, int64_t total_q, int64_t total_kv,
                                           int64_t num_q_heads, int64_t num_kv_heads,
