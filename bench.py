@@ -761,10 +761,12 @@ def hbm_read_probe(gib: int = 4, reps: int = 5):
 
 def mfma_rate_probe():
     """Sustained v_mfma_f32_32x32x16_bf16 rate of the whole chip on register-resident operands,
-    nothing else running: all-zero operands and N(0,1) operands that change every instruction.
-    The board lowers its shader clock to hold its power limit and MFMA power grows with the
-    number of toggling operand bits, so the second figure is context for the prefill number;
-    `roofline.frac` stays the fraction of the datasheet peak."""
+    nothing else running: all-zero operands and N(0,1) operands that change every instruction;
+    then the random stream with the A operand of every instruction read from LDS (1 KB per MFMA,
+    the way the attention kernels receive K and V).  The board lowers its shader clock to hold
+    its power limit and MFMA power grows with the number of toggling operand bits, so the
+    second and third figures are context for the prefill number; `roofline.frac` stays the
+    fraction of the datasheet peak."""
     import ctypes
 
     lib = _probe_lib()
@@ -772,11 +774,11 @@ def mfma_rate_probe():
     lib.msgl_probe_mfma_rate.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_double),
                                          ctypes.POINTER(ctypes.c_double)]
     out = {"unit": "TFLOP/s", "kernel": "back-to-back v_mfma_f32_32x32x16_bf16, 4 waves per CU"}
-    for name, mode in (("zero_operands", 0), ("random_operands", 1)):
+    for name, mode in (("zero_operands", 0), ("random_operands", 1), ("random_operands_a_from_lds", 2)):
         tf, ghz = ctypes.c_double(0), ctypes.c_double(0)
         rc = lib.msgl_probe_mfma_rate(mode, 40000, ctypes.byref(tf), ctypes.byref(ghz))
         if rc != 0:
-            return None
+            return None if mode < 2 else out
         out[name] = tf.value
         out[name + "_shader_ghz"] = ghz.value
         log(f"[mfma probe] {name}: {tf.value:.0f} TFLOP/s at {ghz.value:.2f} GHz")
@@ -909,6 +911,9 @@ def main():
                 # the same MFMA instruction issued back to back on random operands, on this box,
                 # now: what the board sustains under its power limit
                 result["prefill"]["frac_of_measured_mfma_rate"] = pre["achieved_TFLOPs"] / probe["random_operands"]
+            if probe and probe.get("random_operands_a_from_lds"):
+                result["prefill"]["frac_of_measured_lds_fed_mfma_rate"] = (
+                    pre["achieved_TFLOPs"] / probe["random_operands_a_from_lds"])
     if not args.no_mfma_probe:
         result["hbm_read_probe"] = hbm_read_probe()
     if not args.no_metadata:

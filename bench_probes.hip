@@ -7,7 +7,7 @@
 // many operand bits toggle, so the rate is measured for all-zero operands and for operands
 // drawn from N(0,1) that change with every instruction.  The second figure is the ceiling a
 // bf16 attention kernel on random data is measured against; the datasheet peak assumes the
-// boost clock.
+// boost clock.  A third run feeds the A operand of every instruction from LDS.
 //
 // (2) What a plain streaming read sustains: every lane reads 16 bytes per load, consecutive
 // lanes consecutive addresses, a grid-stride loop over a buffer far larger than the 256 MB
@@ -72,6 +72,58 @@ __global__ __launch_bounds__(256) void mfma_rate_kernel(int random_operands, int
 }
 
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
+// The same stream with the A operand of every MFMA read from LDS (16 bytes per lane, 1 KB per
+// instruction, conflict-free), the way an attention kernel receives its K and V tiles: what the
+// matrix pipe sustains when operand delivery draws from the same power budget.  Eight waves per CU
+// (two per SIMD, as in the extend kernel): one wave's LDS latency hides behind the other's MFMAs.
+__global__ __launch_bounds__(512) void mfma_lds_rate_kernel(int iters, float* sink, long long* clocks) {
+  __shared__ __attribute__((aligned(16))) u32x4_t tiles[8 * 16 * 64];  // 128 KB: 16 operands per wave
+  f32x16_t acc[4];
+  for (int a = 0; a < 4; ++a)
+    for (int i = 0; i < 16; ++i) acc[a][i] = 0.f;
+  bf16x8_t bv[8];
+  const uint32_t tid = blockIdx.x * 512 + threadIdx.x;
+  for (int r = 0; r < 8; ++r)
+    for (int i = 0; i < 8; ++i) bv[r][i] = (__bf16)draw(tid * 257 + r * 29 + i + 1000);
+  for (int t = threadIdx.x; t < 8 * 16 * 64; t += 512) {
+    bf16x8_t v;
+    for (int i = 0; i < 8; ++i) v[i] = (__bf16)draw((blockIdx.x * 8192 + t) * 131 + i);
+    tiles[t] = __builtin_bit_cast(u32x4_t, v);
+  }
+  __syncthreads();
+  const u32x4_t* mine = tiles + (threadIdx.x >> 6) * (16 * 64) + (threadIdx.x & 63);
+  const long long c0 = clock64(), w0 = wall_clock64();
+  // the operands of one iteration are requested while the MFMAs of the one before run
+  bf16x8_t av[2][8];
+#pragma unroll
+  for (int r = 0; r < 8; ++r) av[0][r] = __builtin_bit_cast(bf16x8_t, mine[r * 64]);
+  for (int it = 0; it < iters; it += 2) {
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+#pragma unroll
+      for (int r = 0; r < 8; ++r) av[half ^ 1][r] = __builtin_bit_cast(bf16x8_t, mine[((half ^ 1) * 8 + r) * 64]);
+#pragma unroll
+      for (int r = 0; r < 8; ++r)
+        acc[r & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[half][r], bv[r], acc[r & 3], 0, 0, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);  // the 8 LDS reads first
+      __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);  // then the 8 MFMAs
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if ((it & 255) == 254)  // keep the sums finite
+      for (int a = 0; a < 4; ++a)
+        for (int i = 0; i < 16; ++i) acc[a][i] *= 1e-3f;
+  }
+  const long long c1 = clock64(), w1 = wall_clock64();
+  float s = 0.f;
+  for (int a = 0; a < 4; ++a)
+    for (int i = 0; i < 16; ++i) s += acc[a][i];
+  sink[tid] = s;
+  if (threadIdx.x == 0) {
+    clocks[blockIdx.x * 2] = c1 - c0;
+    clocks[blockIdx.x * 2 + 1] = w1 - w0;
+  }
+}
 
 __global__ __launch_bounds__(256) void hbm_read_kernel(const u32x4_t* __restrict__ src, size_t n_vec,
                                                        uint32_t* sink) {
@@ -142,7 +194,9 @@ extern "C" __attribute__((visibility("default"))) int msgl_probe_hbm_read(size_t
   return (int)e;
 }
 
-// Runs the probe on the current device (blocking).  tflops: achieved MFMA rate; shader_ghz:
+// Runs the probe on the current device (blocking).  random_operands: 0 all-zero operands in
+// registers, 1 random operands in registers, 2 random operands with A read from LDS for every
+// instruction.  tflops: achieved MFMA rate; shader_ghz:
 // shader clock during the run (cycle counter against the 100 MHz wall counter).
 // Returns 0, or a hipError_t value.
 extern "C" __attribute__((visibility("default"))) int msgl_probe_mfma_rate(int random_operands,
@@ -155,7 +209,7 @@ extern "C" __attribute__((visibility("default"))) int msgl_probe_mfma_rate(int r
   if (e != hipSuccess) return (int)e;
   float* sink = nullptr;
   long long* clocks = nullptr;
-  e = hipMalloc(&sink, (size_t)cus * 256 * sizeof(float));
+  e = hipMalloc(&sink, (size_t)cus * 512 * sizeof(float));
   if (e != hipSuccess) return (int)e;
   e = hipMalloc(&clocks, (size_t)cus * 2 * sizeof(long long));
   if (e != hipSuccess) {
@@ -165,16 +219,25 @@ extern "C" __attribute__((visibility("default"))) int msgl_probe_mfma_rate(int r
   hipEvent_t t0, t1;
   (void)hipEventCreate(&t0);
   (void)hipEventCreate(&t1);
-  hipLaunchKernelGGL(mfma_rate_kernel, dim3(cus), dim3(256), 0, 0, random_operands, iters / 10 + 1, sink, clocks);
-  (void)hipEventRecord(t0, 0);
-  hipLaunchKernelGGL(mfma_rate_kernel, dim3(cus), dim3(256), 0, 0, random_operands, iters, sink, clocks);
-  (void)hipEventRecord(t1, 0);
+  if (random_operands == 2) {  // random operands, A through LDS
+    iters /= 2;  // eight waves per CU share the pipe
+    hipLaunchKernelGGL(mfma_lds_rate_kernel, dim3(cus), dim3(512), 0, 0, iters / 10 + 1, sink, clocks);
+    (void)hipEventRecord(t0, 0);
+    hipLaunchKernelGGL(mfma_lds_rate_kernel, dim3(cus), dim3(512), 0, 0, iters, sink, clocks);
+    (void)hipEventRecord(t1, 0);
+  } else {
+    hipLaunchKernelGGL(mfma_rate_kernel, dim3(cus), dim3(256), 0, 0, random_operands, iters / 10 + 1, sink, clocks);
+    (void)hipEventRecord(t0, 0);
+    hipLaunchKernelGGL(mfma_rate_kernel, dim3(cus), dim3(256), 0, 0, random_operands, iters, sink, clocks);
+    (void)hipEventRecord(t1, 0);
+  }
   e = hipEventSynchronize(t1);
   float ms = 0.f;
   (void)hipEventElapsedTime(&ms, t0, t1);
   long long c[2] = {0, 1};
   (void)hipMemcpy(c, clocks, sizeof(c), hipMemcpyDeviceToHost);
-  *tflops = (double)cus * 4.0 * iters * 8.0 * 32768.0 / (ms * 1e-3) / 1e12;
+  const double waves = random_operands == 2 ? 8.0 : 4.0;
+  *tflops = (double)cus * waves * iters * 8.0 * 32768.0 / (ms * 1e-3) / 1e12;
   *shader_ghz = (double)c[0] / (double)c[1] * 0.1;
   (void)hipEventDestroy(t0);
   (void)hipEventDestroy(t1);
