@@ -719,7 +719,7 @@ PROBE_LIB = os.path.join(ROOT, "bench_probes.so")
 
 
 def build_probes(force: bool = False) -> str:
-    """Compile bench_probes.hip (the two measurement aids below) into bench_probes.so beside this
+    """Compile bench_probes.hip (the measurement aids below) into bench_probes.so beside this
     file.  hipcc cross-compiles for gfx950, so this also runs where there is no GPU."""
     import subprocess
 
@@ -805,7 +805,7 @@ def main():
                     help="skip the figures of the kernels either side of the path: on-device metadata "
                          "build (slot table -> CSR arrays) and fused q/k norm + rope + KV-store")
     ap.add_argument("--no-mfma-probe", action="store_true",
-                    help="skip the two measurement aids: the matrix pipe's sustained rate on zero "
+                    help="skip the measurement aids: the matrix pipe's sustained rate on zero "
                          "and on random operands, and the rate of a plain streaming read of 4 GiB")
     ap.add_argument("--cpu-flops", type=float, default=3e11,
                     help="flop budget of the CPU baseline sample per shape")

@@ -1,4 +1,4 @@
-// Two measurements that bench.py reports beside the attention figures; benchmarking aids, built
+// Measurements that bench.py reports beside the attention figures; benchmarking aids, built
 // into bench_probes.so beside bench.py, not part of the paged-attention library.
 //
 // (1) What the matrix pipe sustains on this board when nothing else runs: back-to-back
