@@ -315,6 +315,10 @@ MSGL_API int msgl_gdn_state_inplace(const void* q, const void* k, const void* v,
 #define MSGL_TUNE_PREFILL_GANGS 8
 #define MSGL_TUNE_CLOCK_PROBE 9
 MSGL_API int msgl_set_tuning(int32_t knob, int64_t value);
+/* The value the calling thread last set for `knob` (0 if it never did): what its launches and
+ * workspace queries use.  Makes the per-thread scope observable: a value set on another thread
+ * does not show here.  No counterpart in the reference. */
+MSGL_API int msgl_get_tuning(int32_t knob, int64_t* value);
 
 #ifdef __cplusplus
 }

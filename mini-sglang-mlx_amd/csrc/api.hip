@@ -17,6 +17,8 @@ thread_local int64_t t_tune[3] = {0, 0, 0};
 thread_local int64_t t_key_splits = 0;
 thread_local int64_t t_gangs = 0;  // negative: never use gang ranges
 thread_local long long* t_clock_probe = nullptr;
+constexpr int kTuneKnobs = 10;
+thread_local int64_t t_last_set[kTuneKnobs] = {};  // what this thread last passed to msgl_set_tuning
 // launch numbers for the count words of gang ranges (see prefill_gangs()); never 0
 std::atomic<unsigned long long> g_gang_nonce{1};
 
@@ -96,7 +98,15 @@ const char* msgl_strerror(int code) {
   }
 }
 
+int msgl_get_tuning(int32_t knob, int64_t* value) {
+  if (!value) return MSGL_ERR_NULL_POINTER;
+  if (knob < 0 || knob >= kTuneKnobs) return MSGL_ERR_SHAPE;
+  *value = t_last_set[knob];
+  return MSGL_OK;
+}
+
 int msgl_set_tuning(int32_t knob, int64_t value) {
+  if (knob >= 0 && knob < kTuneKnobs) t_last_set[knob] = value;
   if (knob == MSGL_TUNE_SPLITKV_WAVES) {
     msgl::splitkv_set_max_waves((int)value);
     return MSGL_OK;

@@ -24,6 +24,7 @@ SIGNATURES = {
     "msgl_version": (ctypes.c_int, []),
     "msgl_strerror": (ctypes.c_char_p, [ctypes.c_int]),
     "msgl_set_tuning": (ctypes.c_int, [_i32, _i64]),
+    "msgl_get_tuning": (ctypes.c_int, [_i32, ctypes.POINTER(ctypes.c_int64)]),
     "msgl_store_kv_cache": (
         ctypes.c_int,
         [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _vp]),
@@ -123,3 +124,12 @@ def set_tuning(knob: int, value: int) -> None:
     rc = load().msgl_set_tuning(int(knob), int(value))
     if rc != 0:
         raise ValueError(f"msgl_set_tuning({knob}, {value}): {strerror(rc)}")
+
+
+def get_tuning(knob: int) -> int:
+    """What the calling thread last set for `knob` (knobs are per host thread)."""
+    out = ctypes.c_int64(0)
+    rc = load().msgl_get_tuning(int(knob), ctypes.byref(out))
+    if rc != 0:
+        raise ValueError(f"msgl_get_tuning({knob}): {strerror(rc)}")
+    return out.value

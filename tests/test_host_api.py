@@ -322,3 +322,39 @@ def test_validation_is_off_unless_asked_for(monkeypatch):
     assert mk._checks_on(False) is False  # the call's own word wins
     monkeypatch.setenv("MSGL_DEBUG_CHECKS", "0")
     assert mk._checks_on(None) is False
+
+
+def test_tuning_knobs_are_per_host_thread():
+    """msgl_set_tuning acts on the calling thread only; msgl_get_tuning shows what a thread's own
+    launches and workspace queries use."""
+    import threading
+
+    from mini_sglang_amd_kernel import _lib
+
+    lib = _lib.load()
+    cfg3 = (8, 4096, 8 * 8704, 32, 8, 128, 512)
+    with_gangs = lib.msgl_paged_prefill_workspace_bytes(*cfg3)
+    assert with_gangs > 0
+    _lib.set_tuning(_lib.TUNE_PREFILL_GANGS, -1)
+    try:
+        assert _lib.get_tuning(_lib.TUNE_PREFILL_GANGS) == -1
+        assert lib.msgl_paged_prefill_workspace_bytes(*cfg3) == 0
+        seen = {}
+
+        def other():
+            seen["knob"] = _lib.get_tuning(_lib.TUNE_PREFILL_GANGS)
+            seen["bytes"] = lib.msgl_paged_prefill_workspace_bytes(*cfg3)
+            _lib.set_tuning(_lib.TUNE_PREFILL_KEY_SPLITS, 3)
+            seen["own"] = _lib.get_tuning(_lib.TUNE_PREFILL_KEY_SPLITS)
+
+        t = threading.Thread(target=other)
+        t.start()
+        t.join()
+        assert seen == {"knob": 0, "bytes": with_gangs, "own": 3}
+        assert _lib.get_tuning(_lib.TUNE_PREFILL_KEY_SPLITS) == 0  # the other thread's value stayed there
+    finally:
+        _lib.set_tuning(_lib.TUNE_PREFILL_GANGS, 0)
+    assert _lib.get_tuning(_lib.TUNE_PREFILL_GANGS) == 0
+    out = __import__("ctypes").c_int64(5)
+    assert lib.msgl_get_tuning(99, __import__("ctypes").byref(out)) == -9
+    assert lib.msgl_get_tuning(0, None) == -1
