@@ -242,3 +242,48 @@ def test_random_decode_half_precision_and_strides(gpu, seed):
         assert_close_bf16(got, want, what, max_tol=5e-3, mean_tol=4e-4)
     else:
         assert_close_bf16(got, want, what)
+
+
+@pytest.mark.parametrize("seed", range(24 * _SCALE))
+def test_random_forced_gang_ranges(gpu, seed):
+    """Extends of 2, 4, 8 or 16 query blocks per (request, kv head) forced into gang ranges
+    (head_dim 128): random unit lengths, ragged extends, requests with fewer query blocks than the
+    launch, causal and cross masks; against the oracle and against one workgroup per query block."""
+    from mini_sglang_amd_kernel import _lib
+
+    rng = random.Random(7000 + seed)
+    n_kv = rng.choice([8, 8, 4])
+    group = rng.choice([1, 2, 4, 8])
+    batch = rng.randrange(1, 7)
+    if (batch * n_kv) % 8:
+        batch += 1  # whole (request, kv head) units per XCD
+    n_qblk = rng.choice([2, 2, 4, 4, 8, 16])
+    rows = rng.randrange((n_qblk - 1) * 256 + 1, n_qblk * 256 + 1)
+    extend = max(1, (rows + group - 1) // group)
+    while (extend * group + 255) // 256 != n_qblk:
+        extend -= 1
+    ext = [extend] + [extend if rng.random() < 0.6 else rng.randrange(1, extend + 1) for _ in range(batch - 1)]
+    rng.shuffle(ext)
+    kv = [(rng.choice([0, 1, 63, 64, 65, 700, 2048]) if rng.random() < 0.4 else rng.randrange(0, 5000)) + e
+          for e in ext]
+    is_cross = rng.random() < 0.3
+    wl = build_workload("fuzz", "prefill", seed=seed, n_q=n_kv * group, n_kv=n_kv, head_dim=128,
+                        page_size=rng.choice([1, 16]), kv_lens=kv, extend_lens=ext,
+                        pool_factor=rng.choice([1.0, 1.5]), store_new=rng.random() < 0.5,
+                        is_cross_attention=is_cross)
+    what = f"fuzz gang ranges seed={seed} heads={n_kv * group}/{n_kv} ext={ext} kv={kv} cross={is_cross}"
+    print(what, flush=True)
+    lib = _lib.load()
+    try:
+        _lib.set_tuning(_lib.TUNE_PREFILL_GANGS, 1)
+        need = lib.msgl_paged_prefill_workspace_bytes(batch, sum(ext), sum(kv), n_kv * group, n_kv, 128, max(ext))
+        assert need > 0, "the shape was meant to take gang ranges: " + what
+        got, _ = run_gpu(wl, gpu)
+        _lib.set_tuning(_lib.TUNE_PREFILL_GANGS, -1)
+        plain, _ = run_gpu(wl, gpu)
+    finally:
+        _lib.set_tuning(_lib.TUNE_PREFILL_GANGS, 0)
+    want, _ = run_oracle(wl)
+    assert_close_bf16(got, want, what)
+    assert_close_bf16(got, plain.float(), what + " (against one workgroup per query block)", max_tol=8e-3,
+                      mean_tol=4e-4)
