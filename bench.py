@@ -785,6 +785,31 @@ def mfma_rate_probe():
     return out
 
 
+def issue_rate_probes():
+    """LDS read rates and the issue rates of MFMA and VALU work on one and two waves per SIMD
+    (bench_probes.hip): the machine figures that the extend kernels' schedules are read against."""
+    import ctypes
+
+    lib = _probe_lib()
+    lib.msgl_probe_issue_rates.restype = ctypes.c_int
+    lib.msgl_probe_issue_rates.argtypes = [ctypes.POINTER(ctypes.c_double), ctypes.c_int]
+    out = (ctypes.c_double * 10)()
+    if lib.msgl_probe_issue_rates(out, 10) != 0:
+        return None
+    res = {
+        "lds_bytes_per_clk_per_cu": {"ds_read_b128": out[0], "ds_read_b64_tr_b16": out[1]},
+        "simd_cycles_per_mfma_one_wave_per_simd": {"valu_0": out[2], "valu_4": out[3], "valu_8": out[4], "valu_16": out[5]},
+        "simd_cycles_per_mfma_two_waves_per_simd": {"valu_0": out[6], "valu_8": out[7], "valu_16": out[8],
+                                                    "valu_4_exp_1": out[9]},
+    }
+    log(f"[issue probe] LDS per CU and clock: ds_read_b128 {out[0]:.0f} B, ds_read_b64_tr_b16 {out[1]:.0f} B")
+    log("[issue probe] SIMD cycles per v_mfma_f32_32x32x16_bf16 with K v_fma_f32 behind each, one wave per "
+        f"SIMD: K=0 {out[2]:.1f}  K=4 {out[3]:.1f}  K=8 {out[4]:.1f}  K=16 {out[5]:.1f}; two waves per SIMD "
+        f"(first start to last end): K=0 {out[6]:.1f}  K=8 {out[7]:.1f}  K=16 {out[8]:.1f}  "
+        f"K=4 and one v_exp_f32 {out[9]:.1f}")
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -807,6 +832,8 @@ def main():
     ap.add_argument("--no-mfma-probe", action="store_true",
                     help="skip the measurement aids: the matrix pipe's sustained rate on zero "
                          "and on random operands, and the rate of a plain streaming read of 4 GiB")
+    ap.add_argument("--issue-probes", action="store_true",
+                    help="also measure LDS read rates and MFMA / VALU issue rates (a second of GPU time)")
     ap.add_argument("--cpu-flops", type=float, default=3e11,
                     help="flop budget of the CPU baseline sample per shape")
     args = ap.parse_args()
@@ -916,6 +943,8 @@ def main():
                     pre["achieved_TFLOPs"] / probe["random_operands_a_from_lds"])
     if not args.no_mfma_probe:
         result["hbm_read_probe"] = hbm_read_probe()
+    if args.issue_probes:
+        result["issue_probes"] = issue_rate_probes()
     if not args.no_metadata:
         result["qk_norm_rope_store"] = run_norm_rope_store(dev, args.steps, args.warmup,
                                                            not args.no_cpu_baseline)

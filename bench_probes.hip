@@ -142,7 +142,148 @@ __global__ __launch_bounds__(256) void hbm_read_kernel(const u32x4_t* __restrict
   if (x == 0x9e3779b9u) sink[0] = x;  // never true for the fill pattern; keeps the loads alive
 }
 
+// (4) Rates behind the kernels' schedules, in shader cycles counted by one workgroup per launch:
+// what LDS delivers per CU and clock to eight waves that do nothing but read (16-byte reads, and
+// the transposing 8-byte reads that feed V to the matrix pipe, in the extend kernels' address
+// pattern), and how a wave's VALU work shares the issue port with its MFMAs (one MFMA followed by
+// K independent v_fma_f32, one or two waves per SIMD).
+typedef short s16x4_t __attribute__((ext_vector_type(4)));
+#define PROBE_LDS(T, a) ((__attribute__((address_space(3))) T*)(uintptr_t)(a))
+template <int MODE>  // 0: ds_read_b128, consecutive lanes consecutive; 1: ds_read_b64_tr_b16
+__global__ __launch_bounds__(512) void lds_rate_kernel(long long* out, uint32_t* sink, int iters) {
+  __shared__ __attribute__((aligned(16))) unsigned char tile[65536];
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  for (int i = threadIdx.x; i < 65536 / 4; i += 512) reinterpret_cast<uint32_t*>(tile)[i] = mix(i);
+  __syncthreads();
+  uint32_t addr = (uint32_t)(uintptr_t)PROBE_LDS(unsigned char, tile);
+  if (MODE == 0) addr += lane * 16 + w * 1024;
+  else addr += ((lane & 15) >> 2) * 1088 + ((lane >> 4) & 1) * 32 + (lane & 3) * 8 + (lane >> 5) * 4 * 1088 + w * 64;
+  u32x4_t acc = {0u, 0u, 0u, 0u};
+  const long long t0 = clock64();
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      if (MODE == 1) {
+        const s16x4_t v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(PROBE_LDS(s16x4_t, addr + u * 64));
+        acc[0] ^= (uint32_t)v[0];
+        acc[1] ^= (uint32_t)v[2];
+      } else {
+        u32x4_t v;  // (through asm: a plain read of a loop-invariant address would be hoisted)
+        asm volatile("ds_read_b128 %0, %1" : "=v"(v) : "v"(addr + u * 32) : "memory");
+        asm volatile("s_waitcnt lgkmcnt(4)" : "+v"(v));
+        acc ^= v;
+      }
+    }
+  }
+  const long long t1 = clock64();
+  if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x9e3779b9u) sink[0] = acc[0];
+  if ((threadIdx.x & 63) == 0 && blockIdx.x == 0) {  // per wave: see issue_rate_kernel
+    out[2 * w] = t0;
+    out[2 * w + 1] = t1;
+  }
+}
+
+template <int K, int WAVES, int E = 0>  // E: v_exp_f32 per MFMA beside the K v_fma_f32
+__global__ __launch_bounds__(WAVES * 64) void issue_rate_kernel(long long* out, float* sink, int iters) {
+  f32x16_t acc[4];
+  for (int a = 0; a < 4; ++a)
+    for (int i = 0; i < 16; ++i) acc[a][i] = 0.f;
+  bf16x8_t av, bv;
+  for (int i = 0; i < 8; ++i) {
+    av[i] = (__bf16)(threadIdx.x * 0.001f + i);
+    bv[i] = (__bf16)(i * 0.5f - threadIdx.x * 0.002f);
+  }
+  float f[8];
+  for (int i = 0; i < 8; ++i) f[i] = threadIdx.x + i;
+  const float m = 1.0001f, c = 0.5f;
+  const long long t0 = clock64();
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      acc[a] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, bv, acc[a], 0, 0, 0);
+#pragma unroll
+      for (int j = 0; j < K; ++j) asm volatile("v_fma_f32 %0, %0, %1, %2" : "+v"(f[j & 7]) : "v"(m), "v"(c));
+#pragma unroll
+      for (int j = 0; j < E; ++j) asm volatile("v_exp_f32 %0, %0" : "+v"(f[(j + 5) & 7]));
+    }
+  }
+  const long long t1 = clock64();
+  float s = 0.f;
+  for (int a = 0; a < 4; ++a)
+    for (int i = 0; i < 16; ++i) s += acc[a][i];
+  for (int i = 0; i < 8; ++i) s += f[i];
+  sink[blockIdx.x * WAVES * 64 + threadIdx.x] = s;
+  // every wave of workgroup 0 leaves its own start and end: with two waves on a SIMD the older
+  // one wins the arbitration and runs at the rate of a lone wave, so one wave's time says nothing
+  if ((threadIdx.x & 63) == 0 && blockIdx.x == 0) {
+    out[2 * (threadIdx.x >> 6)] = t0;
+    out[2 * (threadIdx.x >> 6) + 1] = t1;
+  }
+}
+
 }  // namespace
+
+// Runs the probes of (4) on the current device (blocking).  out[0], out[1]: LDS bytes per clock and
+// CU for ds_read_b128 and ds_read_b64_tr_b16; out[2..5]: cycles per MFMA and SIMD with K = 0, 4, 8,
+// 16 v_fma_f32 behind each MFMA, one wave per SIMD; out[6..8]: the same with K = 0, 8, 16, two
+// waves per SIMD (from the first start to the last end of the workgroup's waves, per MFMA of one
+// SIMD); out[9]: two waves per SIMD, four v_fma_f32 and one v_exp_f32 per MFMA, the extend kernel's
+// mix.  n_out must be at least 10.  Returns 0 or a hipError_t value.
+extern "C" __attribute__((visibility("default"))) int msgl_probe_issue_rates(double* out, int n_out) {
+  if (!out || n_out < 10) return (int)hipErrorInvalidValue;
+  int dev = 0, cus = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+  if (e != hipSuccess) return (int)e;
+  long long* clk = nullptr;
+  float* sink = nullptr;
+  e = hipMalloc(&clk, 16 * sizeof(long long));
+  if (e != hipSuccess) return (int)e;
+  e = hipMalloc(&sink, (size_t)cus * 512 * sizeof(float));
+  if (e != hipSuccess) {
+    (void)hipFree(clk);
+    return (int)e;
+  }
+  auto span = [&](int waves) {  // first start to last end over the waves of workgroup 0
+    long long h[16] = {0};
+    if (hipDeviceSynchronize() != hipSuccess) return 0.0;
+    (void)hipMemcpy(h, clk, sizeof(h), hipMemcpyDeviceToHost);
+    long long lo = h[0], hi = h[1];
+    for (int w = 1; w < waves; ++w) {
+      lo = h[2 * w] < lo ? h[2 * w] : lo;
+      hi = h[2 * w + 1] > hi ? h[2 * w + 1] : hi;
+    }
+    return (double)(hi - lo);
+  };
+  const int lds_iters = 2000, mfma_iters = 20000;
+  const dim3 grid((unsigned)cus);
+  for (int rep = 0; rep < 2; ++rep)  // the second launch is the one read
+    hipLaunchKernelGGL((lds_rate_kernel<0>), grid, dim3(512), 0, 0, clk, (uint32_t*)sink, lds_iters);
+  out[0] = 8.0 * lds_iters * 8 * 1024 / span(8);
+  for (int rep = 0; rep < 2; ++rep)
+    hipLaunchKernelGGL((lds_rate_kernel<1>), grid, dim3(512), 0, 0, clk, (uint32_t*)sink, lds_iters);
+  out[1] = 8.0 * lds_iters * 8 * 512 / span(8);
+#define MSGL_ISSUE_PROBE(slot, K, WAVES)                                                            \
+  for (int rep = 0; rep < 2; ++rep)                                                                 \
+    hipLaunchKernelGGL((issue_rate_kernel<K, WAVES>), grid, dim3(WAVES * 64), 0, 0, clk, sink, mfma_iters); \
+  out[slot] = span(WAVES) / (mfma_iters * 4.0 * (WAVES / 4));
+  MSGL_ISSUE_PROBE(2, 0, 4)
+  MSGL_ISSUE_PROBE(3, 4, 4)
+  MSGL_ISSUE_PROBE(4, 8, 4)
+  MSGL_ISSUE_PROBE(5, 16, 4)
+  MSGL_ISSUE_PROBE(6, 0, 8)
+  MSGL_ISSUE_PROBE(7, 8, 8)
+  MSGL_ISSUE_PROBE(8, 16, 8)
+#undef MSGL_ISSUE_PROBE
+  for (int rep = 0; rep < 2; ++rep)
+    hipLaunchKernelGGL((issue_rate_kernel<4, 8, 1>), grid, dim3(512), 0, 0, clk, sink, mfma_iters);
+  out[9] = span(8) / (mfma_iters * 4.0 * 2);
+  e = hipGetLastError();
+  (void)hipFree(clk);
+  (void)hipFree(sink);
+  return (int)e;
+}
 
 // Reads `bytes` (a multiple of 16; at least 1 GiB is sensible) `reps` times and reports the best
 // and the mean rate in TB/s.  Blocking; allocates and frees its own buffer.  Returns 0 or a
