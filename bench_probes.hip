@@ -142,7 +142,7 @@ __global__ __launch_bounds__(256) void hbm_read_kernel(const u32x4_t* __restrict
   if (x == 0x9e3779b9u) sink[0] = x;  // never true for the fill pattern; keeps the loads alive
 }
 
-// (4) Rates behind the kernels' schedules, in shader cycles counted by one workgroup per launch:
+// (3) Rates behind the kernels' schedules, in shader cycles counted by one workgroup per launch:
 // what LDS delivers per CU and clock to eight waves that do nothing but read (16-byte reads, and
 // the transposing 8-byte reads that feed V to the matrix pipe, in the extend kernels' address
 // pattern), and how a wave's VALU work shares the issue port with its MFMAs (one MFMA followed by
@@ -223,7 +223,7 @@ __global__ __launch_bounds__(WAVES * 64) void issue_rate_kernel(long long* out, 
 
 }  // namespace
 
-// Runs the probes of (4) on the current device (blocking).  out[0], out[1]: LDS bytes per clock and
+// Runs the probes of (3) on the current device (blocking).  out[0], out[1]: LDS bytes per clock and
 // CU for ds_read_b128 and ds_read_b64_tr_b16; out[2..5]: cycles per MFMA and SIMD with K = 0, 4, 8,
 // 16 v_fma_f32 behind each MFMA, one wave per SIMD; out[6..8]: the same with K = 0, 8, 16, two
 // waves per SIMD (from the first start to the last end of the workgroup's waves, per MFMA of one
